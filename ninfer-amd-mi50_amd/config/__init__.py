@@ -1,8 +1,9 @@
 from .base import ConfigError, KeyReader, architecture_name, read_config_json
+from .fopinex import FopinexConfig
 from .getodra import GetodraConfig
 from .options import EngineOptions
 from .qwen2_moe import Qwen2MoeConfig
 from .sosepel import SosepelConfig
 
 __all__ = ["ConfigError", "KeyReader", "architecture_name", "read_config_json",
-           "EngineOptions", "GetodraConfig", "Qwen2MoeConfig", "SosepelConfig"]
+           "EngineOptions", "FopinexConfig", "GetodraConfig", "Qwen2MoeConfig", "SosepelConfig"]

@@ -9,8 +9,14 @@ namespace ninfer {
 // A gated epilogue forms act(x Wg^T) * (x Wu^T) from the two halves of W's rows; the
 // activation is SiLU (SwiGLU) or the tanh form of GELU (GeGLU).
 // kEpilogueReluSq is not gated: every output (after its bias) becomes max(., 0)^2.
-enum Epilogue : int { kEpilogueNone = 0, kEpilogueSwiGLU = 1, kEpilogueGeGLU = 2, kEpilogueReluSq = 3 };
-inline bool epilogue_gated(int e) { return e == kEpilogueSwiGLU || e == kEpilogueGeGLU; }
+// kEpilogueClampedSwish is gated with both halves cut to a range first:
+//   g' = min(g, limit), u' = clamp(u, -limit, limit), output g' sigmoid(alpha g') (u' + 1)
+// with `act_limit` and `act_alpha` of the arguments.
+enum Epilogue : int { kEpilogueNone = 0, kEpilogueSwiGLU = 1, kEpilogueGeGLU = 2, kEpilogueReluSq = 3,
+                      kEpilogueClampedSwish = 4 };
+inline bool epilogue_gated(int e) {
+  return e == kEpilogueSwiGLU || e == kEpilogueGeGLU || e == kEpilogueClampedSwish;
+}
 // What an ungated epilogue makes of an output.
 __device__ __forceinline__ float ungated_output(float v, bool relu_sq) {
   if (!relu_sq) return v;
@@ -22,6 +28,23 @@ __device__ __forceinline__ float ungated_output(float v, bool relu_sq) {
 // 0.5 g (1 + tanh(c (g + 0.044715 g^3))) with c = sqrt(2 / pi), z = 2 c (g + 0.044715 g^3).
 __device__ __forceinline__ float gate_logit(float g, bool gelu) {
   return gelu ? 1.5957691216057308f * (g + 0.044715f * g * g * g) : g;
+}
+
+// What a gated epilogue makes of a gate value g and the other half's u (both after their
+// biases): the activation of g times u, by the epilogue's kind. `fast`: the hardware's
+// exponential and reciprocal (1 ulp) in place of the library's and an IEEE division.
+template <bool FAST>
+__device__ __forceinline__ float gated_output(float g, float u, int epilogue, float limit, float alpha) {
+  float z;
+  if (epilogue == kEpilogueClampedSwish) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit) + 1.f;
+    z = alpha * g;
+  } else {
+    z = gate_logit(g, epilogue == kEpilogueGeGLU);
+  }
+  if (FAST) return g * __builtin_amdgcn_rcpf(1.f + __expf(-z)) * u;
+  return g / (1.f + expf(-z)) * u;
 }
 
 struct GemmArgs {
@@ -58,6 +81,8 @@ struct GemmArgs {
                          // products run 256-row tiles unless told otherwise here)
   int skinny_two;        // few-row grouped products with two feature sets per block: 1 = whenever
                          // the shape allows, -1 = never
+  float act_limit;       // kEpilogueClampedSwish: the range both halves are cut to (> 0)
+  float act_alpha;       // kEpilogueClampedSwish: the factor on the gate inside the sigmoid
 };
 
 // Which rows does tile `ti` of the grouped enumeration cover? Tiles of

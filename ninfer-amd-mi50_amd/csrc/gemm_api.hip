@@ -64,7 +64,7 @@ static int route_by(const GemmArgs& a, const RouteArgs& rt, hipStream_t stream) 
   int rc = ninfer_router_topk(logits, a.ldc, a.M, &rt, stream);
   if (rc) return rc;
   return ninfer_moe_align(rt.ids, a.M * rt.k, rt.E, rt.offsets, rt.order, rt.tiles16,
-                          rt.tiles_big, rt.tile_counts, stream);
+                          rt.tiles_big, rt.tile_counts, rt.weightless, stream);
 }
 
 static int route_check(const GemmArgs& a, const RouteArgs& rt) {
@@ -76,6 +76,8 @@ static int route_check(const GemmArgs& a, const RouteArgs& rt) {
                  "gemm route: score function %d is neither softmax (0) nor sigmoid (1)", rt.score);
   NINFER_REQUIRE(route_groups_ok(rt), "gemm route: %d groups of which %d are open do not fit %d "
                  "experts and k=%d", rt.n_group, rt.topk_group, rt.E, rt.k);
+  NINFER_REQUIRE(route_weightless_ok(rt), "gemm route: %d of %d experts without weights",
+                 rt.weightless, rt.E);
   return 0;
 }
 

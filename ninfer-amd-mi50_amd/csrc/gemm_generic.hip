@@ -110,7 +110,7 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(GemmArgs a) {
       if (SWIGLU) {
         float g = v + (a.bias ? a.bias[n] : 0.f);
         const float u = accu[i][j] + (a.bias ? a.bias[a.N + n] : 0.f);
-        v = g / (1.f + expf(-gate_logit(g, a.epilogue == kEpilogueGeGLU))) * u;
+        v = gated_output<false>(g, u, a.epilogue, a.act_limit, a.act_alpha);
       } else {
         if (a.bias) v += a.bias[n];
         v = ungated_output(v, a.epilogue == kEpilogueReluSq);
@@ -144,6 +144,8 @@ int gemm_check(const GemmArgs& a) {
   NINFER_REQUIRE(a.groups >= 1, "gemm: groups=%d must be >= 1", a.groups);
   NINFER_REQUIRE(a.offsets || a.groups == 1, "gemm: %d groups without offsets", a.groups);
   NINFER_REQUIRE(!a.a_index || a.a_div >= 1, "gemm: a_div=%d must be >= 1", a.a_div);
+  NINFER_REQUIRE(a.epilogue != kEpilogueClampedSwish || (a.act_limit > 0.f && a.act_alpha == a.act_alpha),
+                 "gemm: the clamped gate needs a positive limit (%g) and a factor", a.act_limit);
   NINFER_REQUIRE(a.epilogue == kEpilogueNone || epilogue_gated(a.epilogue) || a.epilogue == kEpilogueReluSq,
                  "gemm: unknown epilogue %d", a.epilogue);
   NINFER_REQUIRE(!(epilogue_gated(a.epilogue) && a.bias && a.offsets),

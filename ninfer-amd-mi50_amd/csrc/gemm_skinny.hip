@@ -237,7 +237,7 @@ __device__ __forceinline__ void skinny_block(const GemmArgs& a, int rows_arg, in
             v += a.bias[col];
             u += a.bias[a.N + col];
           }
-          v = v / (1.f + __expf(-gate_logit(v, a.epilogue == kEpilogueGeGLU))) * u;
+          v = gated_output<true>(v, u, a.epilogue, a.act_limit, a.act_alpha);
         } else {
           if (a.bias) v += a.bias[col];
           v = ungated_output(v, a.epilogue == kEpilogueReluSq);
@@ -376,7 +376,7 @@ __device__ __forceinline__ void skinny_route_block(const GemmArgs& a, const Rout
   }
   __syncthreads();
   align_block(ids_s, T * rt.k, rt.E, rt.offsets, rt.order, rt.tiles16, rt.tiles_big,
-              rt.tile_counts, cnt);
+              rt.tile_counts, cnt, rt.E - rt.weightless);
 }
 
 // The first block is the router's (product `a` and routing `rt`), the others are the tiles of

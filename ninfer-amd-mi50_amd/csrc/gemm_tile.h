@@ -87,8 +87,8 @@ __device__ inline int staged_w_row(int r, int out0, int N) {
 
 // act(g) * u with the hardware's reciprocal (1 ulp) in place of an IEEE division: a tile's
 // epilogue forms 128 of them per lane, and the division is ten instructions each.
-__device__ __forceinline__ float gated_times(float g, float u, bool gelu) {
-  return g * __builtin_amdgcn_rcpf(1.f + __expf(-gate_logit(g, gelu))) * u;
+__device__ __forceinline__ float gated_times(float g, float u, const GemmArgs& a) {
+  return gated_output<true>(g, u, a.epilogue, a.act_limit, a.act_alpha);
 }
 
 __device__ inline void store_quad(float* p, const float (&v)[4]) {
@@ -111,7 +111,6 @@ __device__ inline void write_accumulators(const GemmArgs& a, const f32x16 (&acc)
   TC* C = (TC*)a.C;
   // four features side by side go out in one store when every such group is whole and aligned
   const bool whole_quads = N % 4 == 0 && a.ldc % 4 == 0 && ((uintptr_t)a.C & 15) == 0;
-  const bool gelu = a.epilogue == kEpilogueGeGLU;
   const bool relu_sq = a.epilogue == kEpilogueReluSq;
 #pragma unroll
   for (int jj = 0; jj < FJ; ++jj) {
@@ -134,7 +133,7 @@ __device__ inline void write_accumulators(const GemmArgs& a, const f32x16 (&acc)
               g += a.bias[f0 + r];
               u += a.bias[N + f0 + r];
             }
-            v[r] = gated_times(g, u, gelu);
+            v[r] = gated_times(g, u, a);
           }
           if (whole_quads) {
             if (f0 < N) store_quad(crow + f0, v);
@@ -188,7 +187,6 @@ __device__ inline void write_accumulators_staged(const GemmArgs& a, const f32x16
   static_assert(U >= 2 && U <= 64 && (U & (U - 1)) == 0, "row pieces");
   const int lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
   const int N = a.N;
-  const bool gelu = a.epilogue == kEpilogueGeGLU;
   const bool relu_sq = a.epilogue == kEpilogueReluSq;
 #pragma unroll
   for (int jj = 0; jj < FJ; ++jj) {
@@ -212,7 +210,7 @@ __device__ inline void write_accumulators_staged(const GemmArgs& a, const f32x16
           for (int r = 0; r < 4; ++r) {
             const float g = acc[i][jj][4 * q + r] + bg[r];
             const float u = acc[i + (SWIGLU ? FI / 2 : 0)][jj][4 * q + r] + bu[r];
-            val[r] = (__bf16)gated_times(g, u, gelu);
+            val[r] = (__bf16)gated_times(g, u, a);
           }
         } else {
           float b[4] = {0.f, 0.f, 0.f, 0.f};

@@ -41,6 +41,9 @@ struct RouteArgs {
   int topk_group;    // groups whose experts are candidates
   int group_top;     // a group's score is the sum of its group_top largest (0 or 1: its largest)
   float renorm_eps;  // added to the sum of the chosen scores before the division
+  int weightless;    // the last so many experts have no weights: they are scored, chosen and
+                     // grouped like the others (their rows come last in `order`), but no tile
+                     // is listed for them, so that the grouped products pass their rows over
 };
 
 // A group-limited choice asks: groups of equal size, at most 64 of them, and enough candidates
@@ -51,6 +54,7 @@ inline bool route_groups_ok(const RouteArgs& rt) {
          rt.topk_group <= rt.n_group && (long)rt.topk_group * (rt.E / rt.n_group) >= rt.k &&
          rt.group_top >= 0 && rt.group_top <= rt.E / rt.n_group;
 }
+inline bool route_weightless_ok(const RouteArgs& rt) { return rt.weightless >= 0 && rt.weightless < rt.E; }
 
 constexpr int kMaxExpertsPerLane = 16;  // up to 1024 experts
 // Many rows: the grouping runs as blocks of this many rows side by side (a launch that counts
@@ -249,9 +253,11 @@ __device__ __forceinline__ int route_row(const float* __restrict__ row, const Ro
 // index. Also writes the lists of 16-row and of kGroupedTileRows-row tiles the grouped
 // products walk: {expert, first row, end row, 0} per tile, and their counts.
 // `cnt` is E + 1 ints of LDS; ids may be in LDS or global memory.
+// Experts from `tiled` on (those without weights) get no tiles.
 __device__ inline void align_block(const int* ids, int n, int E, int* __restrict__ offsets,
                             int* __restrict__ order, int* __restrict__ tiles16,
-                            int* __restrict__ tiles_big, int* __restrict__ tile_counts, int* cnt) {
+                            int* __restrict__ tiles_big, int* __restrict__ tile_counts, int* cnt,
+                            int tiled) {
   constexpr int big = kGroupedTileRows;
   for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
   __syncthreads();
@@ -265,7 +271,8 @@ __device__ inline void align_block(const int* ids, int n, int E, int* __restrict
     for (int e0 = 0; e0 < E; e0 += 64) {
       const int e = e0 + lane;
       const int c = e < E ? cnt[e] : 0;
-      const int t16 = (c + 15) / 16, t64 = (c + big - 1) / big;
+      const int ct = e < tiled ? c : 0;
+      const int t16 = (ct + 15) / 16, t64 = (ct + big - 1) / big;
       int ic = c, i16 = t16, i64 = t64;
 #pragma unroll
       for (int off = 1; off < 64; off <<= 1) {
@@ -282,8 +289,8 @@ __device__ inline void align_block(const int* ids, int n, int E, int* __restrict
         cnt[e] = run;
         if (tiles16) {
           int p16 = n16 + i16 - t16, p64 = n64 + i64 - t64;
-          for (int r = run; r < run + c; r += 16) ((int4*)tiles16)[p16++] = make_int4(e, r, run + c, 0);
-          for (int r = run; r < run + c; r += big) ((int4*)tiles_big)[p64++] = make_int4(e, r, run + c, 0);
+          for (int r = run; r < run + ct; r += 16) ((int4*)tiles16)[p16++] = make_int4(e, r, run + c, 0);
+          for (int r = run; r < run + ct; r += big) ((int4*)tiles_big)[p64++] = make_int4(e, r, run + c, 0);
         }
       }
       run0 += __shfl(ic, 63, 64);
@@ -310,7 +317,7 @@ __device__ inline void align_block(const int* ids, int n, int E, int* __restrict
 extern "C" int ninfer_router_topk(const float* logits, int ld, int T, const ninfer::RouteArgs* rt,
                                   hipStream_t stream);
 extern "C" int ninfer_moe_align(const int* ids, int n, int E, int* offsets, int* order,
-                                int* tiles16, int* tiles_big, int* tile_counts,
+                                int* tiles16, int* tiles_big, int* tile_counts, int weightless,
                                 hipStream_t stream);
 // Scores + top-k and the grouping of many rows (T > 16) in three launches whose blocks work
 // side by side; needs rt->parts. Without it (or for few rows) callers run ninfer_router_topk

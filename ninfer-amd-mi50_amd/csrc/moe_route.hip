@@ -16,9 +16,9 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float* __restrict
 __global__ void moe_align_kernel(const int* __restrict__ ids, int n, int E,
                                  int* __restrict__ offsets, int* __restrict__ order,
                                  int* __restrict__ tiles16, int* __restrict__ tiles_big,
-                                 int* __restrict__ tile_counts) {
+                                 int* __restrict__ tile_counts, int tiled) {
   extern __shared__ int cnt[];
-  align_block(ids, n, E, offsets, order, tiles16, tiles_big, tile_counts, cnt);
+  align_block(ids, n, E, offsets, order, tiles16, tiles_big, tile_counts, cnt, tiled);
 }
 
 // Many rows, after the top-k kernel: block b counts the experts that rows
@@ -63,7 +63,8 @@ __global__ __launch_bounds__(1024) void moe_align_parts_kernel(int T, RouteArgs 
     for (int e0 = 0; e0 < E; e0 += 64) {
       const int e = e0 + lane;
       const int c = e < E ? total[e] : 0;
-      const int t16 = (c + 15) / 16, tb = (c + big - 1) / big;
+      const int ct = e < E - rt.weightless ? c : 0;   // experts without weights get no tiles
+      const int t16 = (ct + 15) / 16, tb = (ct + big - 1) / big;
       int ic = c, i16 = t16, ib = tb;
 #pragma unroll
       for (int off = 1; off < 64; off <<= 1) {
@@ -81,8 +82,8 @@ __global__ __launch_bounds__(1024) void moe_align_parts_kernel(int T, RouteArgs 
           rt.offsets[e] = run;
           if (rt.tiles16) {
             int p16 = n16 + i16 - t16, pb = nbig + ib - tb;
-            for (int r = run; r < run + c; r += 16) ((int4*)rt.tiles16)[p16++] = make_int4(e, r, run + c, 0);
-            for (int r = run; r < run + c; r += big) ((int4*)rt.tiles_big)[pb++] = make_int4(e, r, run + c, 0);
+            for (int r = run; r < run + ct; r += 16) ((int4*)rt.tiles16)[p16++] = make_int4(e, r, run + c, 0);
+            for (int r = run; r < run + ct; r += big) ((int4*)rt.tiles_big)[pb++] = make_int4(e, r, run + c, 0);
           }
         }
       }
@@ -121,7 +122,7 @@ __global__ __launch_bounds__(1024) void moe_route_small_kernel(
   }
   __syncthreads();  // what this block wrote above is read below by other threads of this block
   align_block(ids_s ? ids_s : rt.ids, T * k, E, rt.offsets, rt.order, rt.tiles16, rt.tiles_big,
-              rt.tile_counts, cnt);
+              rt.tile_counts, cnt, E - rt.weightless);
 }
 
 }  // namespace ninfer
@@ -143,6 +144,8 @@ static int route_args_check(const char* who, const RouteArgs& rt, int ld) {
   NINFER_REQUIRE(route_groups_ok(rt), "%s: %d groups of which %d are open do not fit %d experts and "
                  "k=%d (equal groups, at most 64, enough candidates)", who, rt.n_group, rt.topk_group,
                  rt.E, rt.k);
+  NINFER_REQUIRE(route_weightless_ok(rt), "%s: %d of %d experts without weights", who, rt.weightless,
+                 rt.E);
   return 0;
 }
 
@@ -166,14 +169,16 @@ extern "C" int ninfer_router_topk(const float* logits, int ld, int T, const Rout
 // 4 ints for each of up to min(n, n / 16 + E) tiles of 16 rows, tiles_big for up
 // to n / kGroupedTileRows + E tall tiles.
 extern "C" int ninfer_moe_align(const int* ids, int n, int E, int* offsets, int* order,
-                                int* tiles16, int* tiles_big, int* tile_counts,
+                                int* tiles16, int* tiles_big, int* tile_counts, int weightless,
                                 hipStream_t stream) {
   NINFER_REQUIRE(n > 0 && E > 0, "moe_align: n=%d E=%d must be positive", n, E);
+  NINFER_REQUIRE(weightless >= 0 && weightless < E, "moe_align: %d of %d experts without weights",
+                 weightless, E);
   NINFER_REQUIRE(E <= 8192, "moe_align: %d experts exceed 8192", E);
   NINFER_REQUIRE((!tiles16) == (!tiles_big) && (!tiles16) == (!tile_counts),
                  "moe_align: tile lists come together or not at all");
   moe_align_kernel<<<1, 1024, (E + 1) * sizeof(int), stream>>>(ids, n, E, offsets, order, tiles16,
-                                                               tiles_big, tile_counts);
+                                                               tiles_big, tile_counts, E - weightless);
   NINFER_LAUNCH_CHECK();
   return 0;
 }

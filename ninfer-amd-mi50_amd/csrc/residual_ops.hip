@@ -93,6 +93,59 @@ __global__ void scaled_sum_add_kernel(float* __restrict__ residual, const T* __r
   residual[t * H + i] += m;
 }
 
+// What the gated sum adds: residual[t,c] += mult (c1(t,c) a[t,c] + c2(t,c) f(t,c)) in 32-bit,
+// with c = sigmoid(g[t,c] + b[c]) from a gate's logits g (rows of the activation dtype) and
+// bias b, or 1 without a gate; f is dense rows, or the weighted sum of a sparse
+// feed-forward's rows sum_j w[t,j] y[t k + j, c], where a choice j with ids[t,j] >= real
+// stands for an expert that hands its input back: its term is w[t,j] xin[t,c].
+struct GatedSumArgs {
+  float* residual;
+  const void* a;        // [T, H] or null
+  const void* g1;       // [T, H] logits of a's gate, or null
+  const float* b1;      // [H] or null
+  const void* dense;    // [T, H] or null
+  const void* y;        // [T k, H] or null
+  const float* w;       // [T, k]
+  const int* ids;       // [T, k] or null (every choice has a row of y)
+  const void* xin;      // [T, H] what the experts read (with ids)
+  const void* g2;       // [T, H] logits of f's gate, or null
+  const float* b2;      // [H] or null
+  int T, H, k, real, dtype;
+  float mult;
+};
+
+template <typename T>
+__global__ void gated_sum_add_kernel(GatedSumArgs p) {
+  const int64_t t = blockIdx.x;
+  const int i = blockIdx.y * blockDim.x + threadIdx.x;
+  const int H = p.H;
+  if (i >= H) return;
+  float m = 0.f;
+  if (p.a) {
+    m = to_f32(((const T*)p.a)[t * H + i]);
+    if (p.g1) m *= 1.f / (1.f + expf(-(to_f32(((const T*)p.g1)[t * H + i]) + (p.b1 ? p.b1[i] : 0.f))));
+  }
+  float f = 0.f;
+  bool has_f = false;
+  if (p.dense) {
+    f = to_f32(((const T*)p.dense)[t * H + i]);
+    has_f = true;
+  } else if (p.y) {
+    const T* y = (const T*)p.y;
+    for (int j = 0; j < p.k; ++j) {
+      const bool back = p.ids && p.ids[t * p.k + j] >= p.real;
+      const float v = back ? to_f32(((const T*)p.xin)[t * H + i]) : to_f32(y[(t * p.k + j) * H + i]);
+      f = fmaf(p.w[t * p.k + j], v, f);
+    }
+    has_f = true;
+  }
+  if (has_f) {
+    if (p.g2) f *= 1.f / (1.f + expf(-(to_f32(((const T*)p.g2)[t * H + i]) + (p.b2 ? p.b2[i] : 0.f))));
+    m += f;
+  }
+  p.residual[t * H + i] += p.mult * m;
+}
+
 // x <- cap * tanh(x / cap), in place (32-bit numbers).
 __global__ void tanh_cap_kernel(float* __restrict__ x, int64_t n, float cap) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -170,6 +223,21 @@ extern "C" int ninfer_scaled_sum_add(float* residual, const void* a, const float
     scaled_sum_add_kernel<bf16><<<grid, 256, 0, stream>>>(
         residual, (const bf16*)a, s1, (const bf16*)dense, (const bf16*)y, w, k,
         (const bf16*)shared, gate, gate_stride, s2, H);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int ninfer_gated_sum_add(const GatedSumArgs* p, hipStream_t stream) {
+  NINFER_REQUIRE(p->T > 0 && p->H > 0, "gated_sum_add: T=%d H=%d must be positive", p->T, p->H);
+  NINFER_REQUIRE(p->dtype == kF32 || p->dtype == kBF16, "gated_sum_add: unknown dtype %d", p->dtype);
+  NINFER_REQUIRE(!(p->dense && p->y), "gated_sum_add: dense rows or a weighted sum, not both");
+  NINFER_REQUIRE(!p->y || (p->w && p->k > 0), "gated_sum_add: a weighted sum needs weights and k=%d > 0", p->k);
+  NINFER_REQUIRE(!p->ids || (p->xin && p->real >= 0), "gated_sum_add: experts that hand their input "
+                 "back need that input");
+  NINFER_REQUIRE(p->mult == p->mult, "gated_sum_add: the multiplier is no number");
+  dim3 grid(p->T, (p->H + 255) / 256);
+  if (p->dtype == kF32) gated_sum_add_kernel<float><<<grid, 256, 0, stream>>>(*p);
+  else gated_sum_add_kernel<bf16><<<grid, 256, 0, stream>>>(*p);
   NINFER_LAUNCH_CHECK();
   return 0;
 }

@@ -5,7 +5,8 @@
 //                  taps - 1 inputs of a request are per-request state (32-bit), so a request
 //                  may be cut into steps anywhere; before a request's start they are zero.
 //   norm_add       x += y rsqrt(mean(y^2) + eps) g, g one number or one per channel.
-//   gated_rmsnorm  out = o rsqrt(mean(o^2) + eps) w sigmoid(g), the norm over the whole row.
+//   gated_rmsnorm  out = o rsqrt(mean(o^2) + eps) w sigmoid(g) (or w g sigmoid(g)), the norm
+//                  over the whole row or over every group of columns (a head's) by itself.
 //
 // All sums are 32-bit and their order depends on the row alone (taps ascending; the block
 // reduction's order depends on the width), never on how a request was cut or on the batch.
@@ -87,7 +88,7 @@ __global__ void norm_add_kernel(float* __restrict__ x, const T* __restrict__ y,
 template <typename T>
 __global__ void gated_rmsnorm_kernel(const float* __restrict__ o, const T* __restrict__ gate,
                                      int gate_stride, const float* __restrict__ w,
-                                     T* __restrict__ out, int N, float eps) {
+                                     T* __restrict__ out, int N, float eps, int silu) {
   __shared__ float red[16];
   const int64_t r = blockIdx.x;
   const float* orow = o + r * N;
@@ -97,8 +98,30 @@ __global__ void gated_rmsnorm_kernel(const float* __restrict__ o, const T* __res
   const float inv = 1.f / sqrtf(ss / (float)N + eps);
   const T* g = gate + r * gate_stride;
   for (int i = threadIdx.x; i < N; i += blockDim.x) {
-    const float sg = 1.f / (1.f + expf(-to_f32(g[i])));
+    const float z = to_f32(g[i]);
+    const float sg = (silu ? z : 1.f) / (1.f + expf(-z));
     out[r * N + i] = from_f32<T>(orow[i] * inv * w[i] * sg);
+  }
+}
+
+// The same with the norm over every group of `group` neighbouring columns by itself (a head's
+// values) and a weight of `group` numbers that all groups share: one wave per (row, group).
+template <typename T>
+__global__ __launch_bounds__(64) void gated_group_rmsnorm_kernel(
+    const float* __restrict__ o, const T* __restrict__ gate, int gate_stride,
+    const float* __restrict__ w, T* __restrict__ out, int N, int group, float eps, int silu) {
+  const int64_t r = blockIdx.x;
+  const int g0 = blockIdx.y * group, lane = threadIdx.x;
+  const float* orow = o + r * N + g0;
+  float ss = 0.f;
+  for (int i = lane; i < group; i += 64) ss = fmaf(orow[i], orow[i], ss);
+  ss = wave_sum(ss);
+  const float inv = 1.f / sqrtf(ss / (float)group + eps);
+  const T* g = gate + r * gate_stride + g0;
+  for (int i = lane; i < group; i += 64) {
+    const float z = to_f32(g[i]);
+    const float sg = (silu ? z : 1.f) / (1.f + expf(-z));
+    out[r * N + g0 + i] = from_f32<T>(orow[i] * inv * w[i] * sg);
   }
 }
 
@@ -154,19 +177,35 @@ extern "C" int ninfer_norm_add(float* x, const void* y, const float* gain, int g
   return 0;
 }
 
+// group 0 (or N): the norm over the whole row with a weight of N numbers; else over every
+// group of `group` columns with a weight of `group` numbers. silu: the gate's factor is
+// g sigmoid(g) instead of sigmoid(g).
 extern "C" int ninfer_gated_rmsnorm(const float* o, const void* gate, int gate_stride,
                                     const float* w, void* out, int T, int N, float eps, int dtype,
-                                    hipStream_t stream) {
+                                    int group, int silu, hipStream_t stream) {
   NINFER_REQUIRE(T > 0 && N > 0 && gate_stride >= N, "gated_rmsnorm: T=%d N=%d gate stride %d", T,
                  N, gate_stride);
   NINFER_REQUIRE(dtype == kF32 || dtype == kBF16, "gated_rmsnorm: unknown dtype %d", dtype);
+  NINFER_REQUIRE(group >= 0 && (group == 0 || N % group == 0),
+                 "gated_rmsnorm: groups of %d columns do not fill rows of %d", group, N);
+  if (group > 0 && group < N) {
+    const dim3 grid(T, N / group);
+    if (dtype == kF32)
+      gated_group_rmsnorm_kernel<float><<<grid, 64, 0, stream>>>(o, (const float*)gate, gate_stride,
+                                                                 w, (float*)out, N, group, eps, silu);
+    else
+      gated_group_rmsnorm_kernel<bf16><<<grid, 64, 0, stream>>>(o, (const bf16*)gate, gate_stride,
+                                                                w, (bf16*)out, N, group, eps, silu);
+    NINFER_LAUNCH_CHECK();
+    return 0;
+  }
   const int block = N >= 1024 ? 1024 : (N + 63) / 64 * 64;
   if (dtype == kF32)
     gated_rmsnorm_kernel<float><<<T, block, 0, stream>>>(o, (const float*)gate, gate_stride, w,
-                                                         (float*)out, N, eps);
+                                                         (float*)out, N, eps, silu);
   else
     gated_rmsnorm_kernel<bf16><<<T, block, 0, stream>>>(o, (const bf16*)gate, gate_stride, w,
-                                                        (bf16*)out, N, eps);
+                                                        (bf16*)out, N, eps, silu);
   NINFER_LAUNCH_CHECK();
   return 0;
 }

@@ -38,7 +38,8 @@ class _GemmArgs(ctypes.Structure):
                 ("epilogue", ctypes.c_int),
                 ("k_parts", ctypes.c_int), ("workspace", ctypes.c_void_p),
                 ("workspace_floats", ctypes.c_int64), ("split_min_bytes", ctypes.c_int64),
-                ("force_kernel", ctypes.c_int), ("skinny_two", ctypes.c_int)]
+                ("force_kernel", ctypes.c_int), ("skinny_two", ctypes.c_int),
+                ("act_limit", ctypes.c_float), ("act_alpha", ctypes.c_float)]
 
 
 class _RouteArgs(ctypes.Structure):
@@ -49,7 +50,7 @@ class _RouteArgs(ctypes.Structure):
                 ("E", ctypes.c_int), ("k", ctypes.c_int), ("renorm", ctypes.c_int),
                 ("score", ctypes.c_int), ("scale", ctypes.c_float), ("n_group", ctypes.c_int),
                 ("topk_group", ctypes.c_int), ("group_top", ctypes.c_int),
-                ("renorm_eps", ctypes.c_float)]
+                ("renorm_eps", ctypes.c_float), ("weightless", ctypes.c_int)]
 
 
 BIG_TILE_ROWS = 256   # rows of a tall tile of the grouped products (the library's kGroupedTileRows)
@@ -60,7 +61,9 @@ ROUTE_ROWS_PER_BLOCK = 1024  # the library's kAlignRowsPerBlock
 ROUTE_MANY_MIN_ROWS = 2048
 _SCORES = {"softmax": 0, "sigmoid": 1}
 # activations of a gated product, by the names config.json gives them -> the library's epilogue
-GATE_ACTS = {"silu": 1, "gelu_pytorch_tanh": 2}
+# ('clamped_swish': g sigmoid(alpha g) (u + 1) with g cut at a limit from above and u to
+# [-limit, limit]; the limit and alpha travel with the call)
+GATE_ACTS = {"silu": 1, "gelu_pytorch_tanh": 2, "clamped_swish": 4}
 # ... and of a plain product: none, or the square of relu on every output
 UNGATED_ACTS = {None: 0, "relu2": 3}
 
@@ -123,6 +126,29 @@ class _DiffAttnArgs(ctypes.Structure):
                 ("scale", ctypes.c_float), ("cap", ctypes.c_float),
                 ("t_coef", ctypes.c_float), ("t_every", ctypes.c_int), ("lam", ctypes.c_float),
                 ("eps", ctypes.c_float), ("out_scale", ctypes.c_float)]
+
+
+class _SigAttnArgs(ctypes.Structure):
+    _fields_ = [("qkv", ctypes.c_void_p), ("kpool", ctypes.c_void_p), ("vpool", ctypes.c_void_p),
+                ("out", ctypes.c_void_p), ("block_table", ctypes.c_void_p),
+                ("positions", ctypes.c_void_p), ("row_seq", ctypes.c_void_p),
+                ("seq_row_start", ctypes.c_void_p), ("head_bias", ctypes.c_void_p),
+                ("mix", ctypes.c_void_p),
+                ("q_stride", ctypes.c_int), ("bt_stride", ctypes.c_int), ("T", ctypes.c_int),
+                ("S", ctypes.c_int), ("Hq", ctypes.c_int), ("Hkv", ctypes.c_int),
+                ("dim", ctypes.c_int), ("vdim", ctypes.c_int), ("page_size", ctypes.c_int),
+                ("dtype", ctypes.c_int), ("max_qlen", ctypes.c_int), ("max_kv_len", ctypes.c_int),
+                ("chunk", ctypes.c_int), ("force_plain", ctypes.c_int),
+                ("single_rows", ctypes.c_int), ("scale", ctypes.c_float)]
+
+
+class _GatedSumArgs(ctypes.Structure):
+    _fields_ = [("residual", ctypes.c_void_p), ("a", ctypes.c_void_p), ("g1", ctypes.c_void_p),
+                ("b1", ctypes.c_void_p), ("dense", ctypes.c_void_p), ("y", ctypes.c_void_p),
+                ("w", ctypes.c_void_p), ("ids", ctypes.c_void_p), ("xin", ctypes.c_void_p),
+                ("g2", ctypes.c_void_p), ("b2", ctypes.c_void_p),
+                ("T", ctypes.c_int), ("H", ctypes.c_int), ("k", ctypes.c_int),
+                ("real", ctypes.c_int), ("dtype", ctypes.c_int), ("mult", ctypes.c_float)]
 
 
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
@@ -405,6 +431,8 @@ class HipOps:
 
     @staticmethod
     def _check_rows_sum(rs, t, h, dtype):
+        _need(getattr(rs, "ids", None) is None, "row sum: rows of experts that hand their input "
+              "back are added by gated_sum_add only")
         _dev(rs.y, "y", dtype, 2)
         _dev(rs.weights, "weights", torch.float32, 2)
         k = rs.weights.shape[1]
@@ -528,7 +556,8 @@ class HipOps:
 
     # ---- products ---------------------------------------------------------------
     def _gemm(self, a, w, c, *, n, k, m, bias=None, offsets=None, a_index=None, c_index=None,
-              a_div=1, groups=1, epilogue=0, w_group_stride=0, tiles=None, only_if_split=False):
+              a_div=1, groups=1, epilogue=0, w_group_stride=0, tiles=None, only_if_split=False,
+              act_limit=0.0, act_alpha=1.0):
         t16 = t64 = tc = None
         if tiles is not None and tiles.tiles16 is not None:
             t16, t64, tc = tiles.tiles16.data_ptr(), tiles.tiles_big.data_ptr(), \
@@ -540,6 +569,7 @@ class HipOps:
         args.force_kernel = self._tune["force_kernel"]
         args.split_min_bytes = self._tune["split_min_bytes"]
         args.skinny_two = self._tune["skinny_two"]
+        args.act_limit, args.act_alpha = float(act_limit), float(act_alpha)
         if only_if_split:
             # a dense product of few dozen rows: the library's unless the kernels here cut it
             # along K (its output tiles alone would not fill the GPU). The one workspace of
@@ -674,7 +704,7 @@ class HipOps:
         _need(act in GATE_ACTS, f"gated product: activation {act!r} is not one of {sorted(GATE_ACTS)}")
         return GATE_ACTS[act]
 
-    def swiglu_linear(self, x, w_gate_up, out, act="silu", bias=None):
+    def swiglu_linear(self, x, w_gate_up, out, act="silu", bias=None, limit=0.0, alpha=1.0):
         """out = act(x Wg^T [+ bg]) * (x Wu^T [+ bu]), Wg = rows [0, I), Wu = rows [I, 2I); act
         is SiLU or the tanh form of GELU (`GATE_ACTS`); `bias` [2I] (32-bit) holds bg, then bu."""
         _dev(x, "x", dims=2)
@@ -687,11 +717,13 @@ class HipOps:
             _dev(bias, "bias", torch.float32, 1)
             _need(bias.shape[0] == 2 * inner, "swiglu_linear: bias has the wrong size")
         self._gemm(x, w_gate_up, out, m=x.shape[0], n=inner, k=x.shape[1],
-                   epilogue=self._gate_epilogue(act), bias=bias)
+                   epilogue=self._gate_epilogue(act), bias=bias, act_limit=limit, act_alpha=alpha)
 
-    def grouped_swiglu(self, x, w_gate_up, offsets, order, top_k, out, tiles=None, act="silu"):
+    def grouped_swiglu(self, x, w_gate_up, offsets, order, top_k, out, tiles=None, act="silu",
+                       limit=0.0, alpha=1.0):
         """out[r] = the gated product (see `swiglu_linear`) of row order[r] // top_k of x by
-        the expert that owns sorted position r."""
+        the expert that owns sorted position r. `offsets` may go on beyond the experts that
+        `w_gate_up` holds (experts without weights, sorted last): their rows are passed over."""
         _dev(x, "x", dims=2)
         _dev(w_gate_up, "w_gate_up", x.dtype, 3)
         _dev(out, "out", x.dtype, 2)
@@ -701,11 +733,11 @@ class HipOps:
         inner = two_i // 2
         n = order.shape[0]
         _need(h == x.shape[1] and two_i == 2 * inner, "grouped_swiglu: weight shape")
-        _need(offsets.shape[0] == e + 1, "grouped_swiglu: offsets size")
+        _need(offsets.shape[0] >= e + 1, "grouped_swiglu: offsets size")
         _need(n == x.shape[0] * top_k and out.shape == (n, inner), "grouped_swiglu: row counts")
         self._gemm(x, w_gate_up, out, m=n, n=inner, k=h, offsets=offsets, a_index=order,
                    a_div=top_k, groups=e, epilogue=self._gate_epilogue(act),
-                   w_group_stride=two_i * h, tiles=tiles)
+                   w_group_stride=two_i * h, tiles=tiles, act_limit=limit, act_alpha=alpha)
 
     def grouped_down(self, h, w_down, offsets, order, out, tiles=None):
         """out[order[r]] = h[r] Wd_e^T for the expert e that owns sorted position r."""
@@ -717,15 +749,16 @@ class HipOps:
         e, hidden, inner = w_down.shape
         n = order.shape[0]
         _need(inner == h.shape[1] and h.shape[0] == n, "grouped_down: input shape")
-        _need(out.shape == (n, hidden) and offsets.shape[0] == e + 1, "grouped_down: shapes")
+        _need(out.shape == (n, hidden) and offsets.shape[0] >= e + 1, "grouped_down: shapes")
         self._gemm(h, w_down, out, m=n, n=hidden, k=inner, offsets=offsets, c_index=order,
                    groups=e, w_group_stride=hidden * inner, tiles=tiles)
 
     # ---- routing ------------------------------------------------------------------
     def _route_args(self, experts, top_k, renorm, ids, wts, r=None, score="softmax",
                     choice_bias=None, scale=1.0, n_group=0, topk_group=0, group_top=1,
-                    renorm_eps=0.0):
+                    renorm_eps=0.0, weightless=0):
         """The router's parameters and the places routing writes, as the library takes them.
+        `weightless`: the last so many experts have no weights (no tiles are listed for them).
         `score`: 'softmax' over all experts or 'sigmoid' of each logit; `choice_bias` [experts]
         is added to the scores for the choice of experts only (the weights are the scores);
         `scale` multiplies every weight, after the renormalisation if there is one; with
@@ -752,7 +785,7 @@ class HipOps:
         args = _RouteArgs(ids.data_ptr(), wts.data_ptr(), offsets, order, t16, t64, tc,
                           _ptr(choice_bias), parts, experts, top_k, 1 if renorm else 0,
                           _SCORES[score], float(scale), int(n_group), int(topk_group),
-                          int(group_top), float(renorm_eps))
+                          int(group_top), float(renorm_eps), int(weightless))
         return args
 
     def router_topk(self, logits, experts, top_k, renorm, ids, wts, score="softmax",
@@ -780,7 +813,7 @@ class HipOps:
               and tiles.tile_counts.shape[0] == 2, "routing: tile lists have the wrong sizes")
         return tiles.tiles16.data_ptr(), tiles.tiles_big.data_ptr(), tiles.tile_counts.data_ptr()
 
-    def moe_align(self, ids, experts, offsets, order, tiles=None):
+    def moe_align(self, ids, experts, offsets, order, tiles=None, weightless=0):
         _dev(ids, "ids", torch.int32)
         _dev(offsets, "offsets", torch.int32, 1)
         _dev(order, "order", torch.int32, 1)
@@ -790,10 +823,11 @@ class HipOps:
         self._ok(self.lib.ninfer_moe_align(
             ctypes.c_void_p(ids.data_ptr()), ids.numel(), experts,
             ctypes.c_void_p(offsets.data_ptr()), ctypes.c_void_p(order.data_ptr()),
-            ctypes.c_void_p(t16), ctypes.c_void_p(t64), ctypes.c_void_p(tc), self._stream()))
+            ctypes.c_void_p(t16), ctypes.c_void_p(t64), ctypes.c_void_p(tc), int(weightless),
+            self._stream()))
 
     def moe_route(self, logits, experts, top_k, renorm, r, score="softmax", choice_bias=None,
-                  scale=1.0, n_group=0, topk_group=0, group_top=1, renorm_eps=0.0):
+                  scale=1.0, n_group=0, topk_group=0, group_top=1, renorm_eps=0.0, weightless=0):
         """Scores + top-k per row (see `_route_args` for the router's parameters) and the
         grouping by expert, into the routing record `r` (ids, weights, offsets, order, tile
         lists): one launch for up to 16 rows (one block does both), two for more (top-k by
@@ -811,7 +845,7 @@ class HipOps:
               and r.offsets.shape[0] == experts + 1 and r.order.shape[0] == t * top_k,
               "moe_route: output sizes")
         rargs = self._route_args(experts, top_k, renorm, r.ids, r.weights, r, score, choice_bias,
-                                 scale, n_group, topk_group, group_top, renorm_eps)
+                                 scale, n_group, topk_group, group_top, renorm_eps, weightless)
         if self._held is not None:
             _need(self._held_route is None, "together(): one routing at most")
             self._held_route = (logits, rargs, (logits, rargs, r, choice_bias))
@@ -829,7 +863,7 @@ class HipOps:
             self._ok(self.lib.ninfer_router_topk(
                 ctypes.c_void_p(logits.data_ptr()), logits.shape[1], t, ctypes.byref(rargs),
                 self._stream()))
-            self.moe_align(r.ids, rargs.E, r.offsets, r.order, tiles=r)
+            self.moe_align(r.ids, rargs.E, r.offsets, r.order, tiles=r, weightless=rargs.weightless)
             return
         self._ok(self.lib.ninfer_moe_route_small(
             ctypes.c_void_p(logits.data_ptr()), logits.shape[1], t, ctypes.byref(rargs),
@@ -934,14 +968,19 @@ class HipOps:
             ctypes.c_void_p(gain.data_ptr()), gain.shape[0], y.shape[0], y.shape[1],
             ctypes.c_float(eps), _DT[y.dtype], self._stream()))
 
-    def gated_rmsnorm(self, o, gate, weight, eps, out):
-        """out = o rsqrt(mean(o^2) + eps) weight sigmoid(gate), the mean over the whole row.
-        o: [T, N] 32-bit; gate: [T, N] columns of a wider row-major tensor (a view)."""
+    def gated_rmsnorm(self, o, gate, weight, eps, out, group=0, gate_act="sigmoid"):
+        """out = o rsqrt(mean(o^2) + eps) weight sigmoid(gate), the mean over the whole row, or
+        with `group` over every group of so many neighbouring columns by itself (`weight` then
+        has `group` numbers, shared by the groups). `gate_act` 'silu': gate sigmoid(gate) in
+        place of sigmoid(gate). o: [T, N] 32-bit; gate: [T, N] columns of a wider row-major
+        tensor (a view)."""
         _dev(o, "o", torch.float32, 2)
         _dev(weight, "weight", torch.float32, 1)
         _dev(out, "out", dims=2)
         t, n = o.shape
-        _need(out.shape == (t, n) and weight.shape[0] == n and out.dtype in _DT,
+        _need(gate_act in ("sigmoid", "silu"), f"gated_rmsnorm: gate activation {gate_act!r}")
+        _need(group >= 0 and (group == 0 or n % group == 0), "gated_rmsnorm: groups do not fill the rows")
+        _need(out.shape == (t, n) and weight.shape[0] == (group or n) and out.dtype in _DT,
               "gated_rmsnorm: shapes")
         _need(gate.is_cuda and gate.dtype == out.dtype and gate.shape == (t, n)
               and gate.stride(1) == 1, "gated_rmsnorm: the gate must be [T, N] columns of rows")
@@ -949,7 +988,8 @@ class HipOps:
             ctypes.c_void_p(o.data_ptr()), ctypes.c_void_p(gate.data_ptr()),
             gate.stride(0) if t > 1 else max(n, gate.stride(0)),
             ctypes.c_void_p(weight.data_ptr()), ctypes.c_void_p(out.data_ptr()), t, n,
-            ctypes.c_float(eps), _DT[out.dtype], self._stream()))
+            ctypes.c_float(eps), _DT[out.dtype], int(group), 1 if gate_act == "silu" else 0,
+            self._stream()))
 
     def lightning_attention(self, qkv, q_off, k_off, v_off, heads, dim, vdim, decay, state, ctx,
                             out):
@@ -1231,6 +1271,129 @@ class HipOps:
             ws = self._workspace(need, qkv.device)
             a.workspace, a.workspace_floats = ws.data_ptr(), ws.numel()
         self._ok(self.lib.ninfer_diff_attention(ctypes.byref(a), self._stream()))
+
+    def gated_sum_add(self, residual, a, g1, b1, f, g2, b2, mult=1.0):
+        """residual += mult (c1 a + c2 f) in 32-bit: a rows [T, H] or None; f rows [T, H], a
+        weighted sum of rows (an object with y, weights and, where some chosen experts hand
+        their input back, ids, real and rows) or None; c = sigmoid(g + b) per row and column
+        from a gate's logits g [T, H] and bias b [H] (32-bit), or 1 where g is None."""
+        _dev(residual, "residual", torch.float32, 2)
+        t, h = residual.shape
+        p = _GatedSumArgs()
+        p.residual, p.T, p.H, p.mult = residual.data_ptr(), t, h, float(mult)
+        dtype = None
+        keep = [residual, a, g1, b1, f, g2, b2]
+        if a is not None:
+            _dev(a, "a", dims=2)
+            _need(a.shape == (t, h) and a.dtype in _DT, "gated_sum_add: a does not fit")
+            dtype = a.dtype
+            p.a = a.data_ptr()
+        if f is not None and hasattr(f, "weights"):
+            dtype = dtype or f.y.dtype
+            _need(getattr(f, "shared", None) is None, "gated_sum_add: no shared expert's rows")
+            k = f.weights.shape[1]
+            _dev(f.y, "y", dtype, 2)
+            _dev(f.weights, "weights", torch.float32, 2)
+            _need(f.y.shape == (t * k, h) and f.weights.shape == (t, k), "gated_sum_add: weighted rows do not fit")
+            p.y, p.w, p.k = f.y.data_ptr(), f.weights.data_ptr(), k
+            if getattr(f, "ids", None) is not None:
+                _dev(f.ids, "ids", torch.int32, 2)
+                _dev(f.rows, "rows", dtype, 2)
+                _need(f.ids.shape == (t, k) and f.rows.shape == (t, h), "gated_sum_add: ids or rows do not fit")
+                p.ids, p.xin, p.real = f.ids.data_ptr(), f.rows.data_ptr(), int(f.real)
+        elif f is not None:
+            dtype = dtype or f.dtype
+            _dev(f, "f", dtype, 2)
+            _need(f.shape == (t, h), "gated_sum_add: f does not fit")
+            p.dense = f.data_ptr()
+        if dtype is None:
+            return
+        for g, b, name in ((g1, b1, "1"), (g2, b2, "2")):
+            if g is None:
+                continue
+            _dev(g, "g" + name, dtype, 2)
+            _need(g.shape == (t, h), f"gated_sum_add: gate {name} does not fit")
+            setattr(p, "g" + name, g.data_ptr())
+            if b is not None:
+                _dev(b, "b" + name, torch.float32, 1)
+                _need(b.shape[0] == h, f"gated_sum_add: bias {name} has the wrong size")
+                setattr(p, "b" + name, b.data_ptr())
+        p.dtype = _DT[dtype]
+        self._ok(self.lib.ninfer_gated_sum_add(ctypes.byref(p), self._stream()))
+        del keep
+
+    def gated_linear_attention(self, qkv, q_off, k_off, v_off, z, heads, dim, vdim, tau, q_scale,
+                               state, ctx, out):
+        """Linear attention with a decay per key channel and token over the rows of each
+        request: S <- diag(alpha) S + k v^T, out = S^T (q q_scale) with alpha =
+        sigmoid(z)^(1 / tau), q, k at the columns q_off, k_off (heads x dim) and v at v_off
+        (heads x vdim) of `qkv`; z: [T, heads * dim] 32-bit. `state` ([slots, >= heads * dim *
+        vdim] 32-bit view) holds every request's S between steps. out: [T, heads * vdim] 32-bit."""
+        _dev(qkv, "qkv", dims=2)
+        _dev(z, "z", torch.float32, 2)
+        _dev(out, "out", torch.float32, 2)
+        t = qkv.shape[0]
+        _need(qkv.dtype in _DT, f"gated_linear_attention: rows of {qkv.dtype}")
+        _need(z.shape == (t, heads * dim) and out.shape == (t, heads * vdim) and ctx.T == t,
+              "gated_linear_attention: shapes")
+        for off, n in ((q_off, heads * dim), (k_off, heads * dim), (v_off, heads * vdim)):
+            _need(0 <= off and off + n <= qkv.shape[1], "gated_linear_attention: columns outside the rows")
+        _need(state.is_cuda and state.dtype == torch.float32 and state.dim() == 2
+              and state.stride(1) == 1 and state.shape[1] >= heads * dim * vdim,
+              "gated_linear_attention: the state must be 32-bit rows of heads * dim * vdim numbers")
+        self._ok(self.lib.ninfer_gated_linear_attention(
+            ctypes.c_void_p(qkv.data_ptr()), qkv.shape[1], q_off, k_off, v_off,
+            ctypes.c_void_p(z.data_ptr()), ctypes.c_float(tau), ctypes.c_float(q_scale),
+            ctypes.c_void_p(state.data_ptr()), ctypes.c_longlong(state.stride(0)),
+            ctypes.c_void_p(out.data_ptr()), ctypes.c_void_p(ctx.seq_row_start.data_ptr()),
+            ctypes.c_void_p(ctx.seq_slots.data_ptr()), t, ctx.S, heads, dim, vdim, _DT[qkv.dtype],
+            self._stream()))
+
+    def sigmoid_attention(self, qkv, k_pool, v_pool, block_table, ctx, heads, kv_heads, dim, vdim,
+                          page_size, scale, chunk, head_bias, mix, out, write_kv=True):
+        """Attention without a softmax over the rows of `qkv` ([T, heads x dim] queries,
+        followed by kv_heads x dim keys and kv_heads x vdim values when `write_kv`: those go
+        into the requests' pages first). The weight of key j for row i of head a is
+        sigmoid((q . k) scale + head_bias[a]) where j <= i and, with chunk > 0,
+        floor(i / chunk) == floor(j / chunk), else 0; with `mix` [heads, heads] the heads'
+        weights are mixed (w'_a = sum_b mix[a, b] w_b); head a applies its weights to the
+        values of kv head a // (heads / kv_heads). out: [T, heads x vdim]."""
+        _dev(qkv, "qkv", dims=2)
+        _need(qkv.dtype in _DT, f"sigmoid_attention: rows of {qkv.dtype}")
+        _dev(k_pool, "k_pool", qkv.dtype, 4)
+        _dev(v_pool, "v_pool", qkv.dtype, 4)
+        _dev(out, "out", qkv.dtype, 2)
+        _dev(block_table, "block_table", torch.int32, 2)
+        t = qkv.shape[0]
+        width = heads * dim + (kv_heads * (dim + vdim) if write_kv else 0)
+        _need(t == ctx.T and qkv.shape[1] == width, "sigmoid_attention: qkv has the wrong shape")
+        _need(out.shape == (t, heads * vdim), "sigmoid_attention: out has the wrong shape")
+        _need(k_pool.shape[1:] == (kv_heads, page_size, dim)
+              and v_pool.shape[1:] == (kv_heads, page_size, vdim)
+              and k_pool.shape[0] == v_pool.shape[0],
+              "sigmoid_attention: pools do not fit the head layout")
+        _need(block_table.shape[0] == ctx.S, "sigmoid_attention: block table rows != requests")
+        a = _SigAttnArgs()
+        a.qkv, a.kpool, a.vpool, a.out = qkv.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), out.data_ptr()
+        a.block_table, a.positions = block_table.data_ptr(), ctx.positions.data_ptr()
+        a.row_seq, a.seq_row_start = ctx.row_seq.data_ptr(), ctx.seq_row_start.data_ptr()
+        if head_bias is not None:
+            _dev(head_bias, "head_bias", torch.float32, 1)
+            _need(head_bias.shape[0] == heads, "sigmoid_attention: one bias per head")
+            a.head_bias = head_bias.data_ptr()
+        if mix is not None:
+            _dev(mix, "mix", torch.float32, 2)
+            _need(mix.shape == (heads, heads), "sigmoid_attention: the mixing matrix is [heads, heads]")
+            a.mix = mix.data_ptr()
+        a.q_stride, a.bt_stride, a.T, a.S = qkv.shape[1], block_table.shape[1], t, ctx.S
+        a.Hq, a.Hkv, a.dim, a.vdim, a.page_size = heads, kv_heads, dim, vdim, page_size
+        a.dtype, a.max_qlen, a.max_kv_len = _DT[qkv.dtype], ctx.max_qlen, ctx.max_kv_len
+        a.chunk, a.scale = int(chunk), float(scale)
+        a.force_plain = 1 if self.force_generic else 0
+        a.single_rows = int(getattr(ctx, "single_rows", 0))
+        if write_kv:
+            self._ok(self.lib.ninfer_sigmoid_kv_write(ctypes.byref(a), self._stream()))
+        self._ok(self.lib.ninfer_sigmoid_attention(ctypes.byref(a), self._stream()))
 
     # ---- sampling -------------------------------------------------------------------
     FEW_TOKENS = 64   # most tokens a row may keep (top_k) for the two-launch sampling path

@@ -4,6 +4,7 @@ from .base import (Block, CacheNeed, CacheView, CallInfo, FeedForward, Mixer, No
 from .block import OutputNormBlock, ParallelBlock, PreNormBlock
 from .diff_attention import DifferentialAttention
 from .embedding import LMHead, TokenEmbedding
+from .gla import GatedLinearAttention
 from .latent_attention import LatentAttention
 from .lightning import LightningAttention
 from .mlp import MLP, SwiGLU
@@ -12,10 +13,12 @@ from .norm import OutputRMSNorm, RMSNorm
 from .rotary import NoPosition, Rotary
 from .reentry import StreamReentry
 from .short_conv import ShortConv
+from .sigmoid_attention import SigmoidAttention
 
 __all__ = ["Attention", "Block", "CacheNeed", "CacheView", "CallInfo", "FeedForward", "Mixer",
            "Norm", "Part", "PendingRows", "PoolSpec", "settle", "PositionEncoding", "StepContext", "WeightBinder", "PreNormBlock",
            "LMHead", "TokenEmbedding", "SwiGLU", "RoutedExperts", "Routing", "SoftmaxTopKRouter", "TopKRouter",
            "SparseMoE", "RMSNorm", "NoPosition", "Rotary", "OutputNormBlock", "OutputRMSNorm",
            "LatentAttention", "LightningAttention", "ShortConv", "ParallelBlock",
-           "DifferentialAttention", "MLP", "StreamReentry"]
+           "DifferentialAttention", "MLP", "StreamReentry", "GatedLinearAttention",
+           "SigmoidAttention"]

@@ -119,14 +119,23 @@ class PendingRows:
     whoever comes next (a norm's kernel adds it on the fly):
     sum_j weights[t, j] * y[t * k + j, :] + sigmoid(gate[t]) * shared[t, :].
     `shared` and `gate` may be None (no such term / factor 1). `gate` is a
-    32-bit view [T] that may be strided."""
+    32-bit view [T] that may be strided. With `ids` ([T, k], the chosen experts), a choice j
+    with ids[t, j] >= `real` stands for an expert without weights that hands its input back:
+    its term is weights[t, j] * rows[t, :] (`rows`: what the experts read), and row t * k + j
+    of y holds nothing."""
     y: torch.Tensor
     weights: torch.Tensor
     shared: Optional[torch.Tensor] = None
     gate: Optional[torch.Tensor] = None
+    ids: Optional[torch.Tensor] = None
+    real: int = 0
+    rows: Optional[torch.Tensor] = None
 
     def add_to(self, ctx: "StepContext", residual: torch.Tensor) -> None:
-        ctx.ops.moe_combine(residual, self.y, self.weights, self.shared, self.gate)
+        if self.ids is not None:
+            ctx.ops.gated_sum_add(residual, None, None, None, self, None, None, 1.0)
+        else:
+            ctx.ops.moe_combine(residual, self.y, self.weights, self.shared, self.gate)
 
 
 def settle(ctx: "StepContext", residual: torch.Tensor, pending) -> Optional[torch.Tensor]:

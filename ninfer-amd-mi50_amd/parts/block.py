@@ -99,48 +99,95 @@ register_part("block", "output_norm", OutputNormBlock)
 
 
 class ParallelBlock(Block):
-    """A block whose sublayers read the same normed rows: h = norm(x), then
-    x += s1 mixer(h) + s2 feed_forward(h), with s1 and s2 one learned factor per column
-    (`mixer_scale`, `ff_scale`: tensor names, None for no factor). `feed_forward` may be None.
-    The sum is formed in 32-bit by one kernel, which also adds up a sparse feed-forward's
-    weighted rows."""
+    """A block whose sublayers run side by side on the same residual: h = norm(x), then
+    x += mult (c1 mixer(h) + c2 feed_forward(h2)), where h2 = h, or ff_norm(x) when the block
+    has a second norm of the same x (`ff_norm`), and c1, c2 are per-column factors:
+    a learned factor per column (`mixer_scale`, `ff_scale`: tensor names, None for no factor),
+    or a gate computed from the sublayer's own input, c = sigmoid(W h + b) per row and column
+    (`mixer_gate`, `ff_gate`: the name of W [size, size]; its bias is that name + ".b").
+    `feed_forward` may be None. The sum is formed in 32-bit by one kernel, which also adds up
+    a sparse feed-forward's weighted rows."""
 
     def __init__(self, norm: Norm, mixer: Mixer, feed_forward: Optional[FeedForward] = None,
-                 mixer_scale: Optional[str] = None, ff_scale: Optional[str] = None, size: int = 0):
+                 mixer_scale: Optional[str] = None, ff_scale: Optional[str] = None, size: int = 0,
+                 ff_norm: Optional[Norm] = None, mult: float = 1.0,
+                 mixer_gate: Optional[str] = None, ff_gate: Optional[str] = None):
+        if (mixer_scale and mixer_gate) or (ff_scale and ff_gate):
+            raise ValueError("a sublayer has a learned factor or a gate, not both")
         self.norm = norm
         self.mixer = mixer
         self.feed_forward = feed_forward
+        self.ff_norm = ff_norm if feed_forward is not None else None
+        self.spare_norm = ff_norm if feed_forward is None else None
+        self.mult = float(mult)
         self.mixer_scale_name = mixer_scale
         self.ff_scale_name = ff_scale if feed_forward is not None else None
         self.spare_scale_name = ff_scale if feed_forward is None else None
+        self.mixer_gate_name = mixer_gate
+        self.ff_gate_name = ff_gate if feed_forward is not None else None
+        self.spare_gate_name = ff_gate if feed_forward is None else None
         self.size = size
         self.mixer_scale: Optional[torch.Tensor] = None
         self.ff_scale: Optional[torch.Tensor] = None
+        self.mixer_gate = self.mixer_gate_bias = self.ff_gate = self.ff_gate_bias = None
 
     def children(self) -> List[Part]:
-        return [p for p in (self.norm, self.mixer, self.feed_forward) if p is not None]
+        return [p for p in (self.norm, self.mixer, self.ff_norm, self.feed_forward) if p is not None]
 
     def tensor_specs(self):
-        return {n: TensorSpec((self.size,), "gain")
-                for n in (self.mixer_scale_name, self.ff_scale_name) if n}
+        specs = {n: TensorSpec((self.size,), "gain")
+                 for n in (self.mixer_scale_name, self.ff_scale_name) if n}
+        for n in (self.mixer_gate_name, self.ff_gate_name):
+            if n:
+                specs[n] = TensorSpec((self.size, self.size))
+                specs[n + ".b"] = TensorSpec((self.size,), "bias")
+        return specs
 
     def unused_tensor_specs(self):
-        # a layer without a feed-forward may still carry the factor of one
+        # a layer without a feed-forward may still carry what belongs to one
+        out = {}
         if self.spare_scale_name:
-            return {self.spare_scale_name: TensorSpec((self.size,), "gain")}
-        return {}
+            out[self.spare_scale_name] = TensorSpec((self.size,), "gain")
+        if self.spare_gate_name:
+            out[self.spare_gate_name] = TensorSpec((self.size, self.size))
+            out[self.spare_gate_name + ".b"] = TensorSpec((self.size,), "bias")
+        if self.spare_norm is not None:
+            out.update(self.spare_norm.all_tensor_specs())
+        return out
 
     def bind(self, w: WeightBinder) -> None:
         if self.mixer_scale_name:
             self.mixer_scale = w.float32(self.mixer_scale_name)
         if self.ff_scale_name:
             self.ff_scale = w.float32(self.ff_scale_name)
+        if self.mixer_gate_name:
+            self.mixer_gate = w.matrix(self.mixer_gate_name)
+            self.mixer_gate_bias = w.float32(self.mixer_gate_name + ".b")
+        if self.ff_gate_name:
+            self.ff_gate = w.matrix(self.ff_gate_name)
+            self.ff_gate_bias = w.float32(self.ff_gate_name + ".b")
+
+    def _gate(self, ctx: StepContext, h, weight):
+        if weight is None:
+            return None
+        g = ctx.empty((h.shape[0], self.size))
+        ctx.ops.linear(h, weight, g)
+        return g
 
     def forward(self, ctx: StepContext, residual, pending, call: CallInfo):
         h = self.norm.forward(ctx, residual, pending)
+        h2 = h
+        if self.ff_norm is not None:
+            h2 = self.ff_norm.forward(ctx, residual, None)
         a = self.mixer.forward(ctx, h, residual, call)
-        f = self.feed_forward.forward(ctx, h, residual) if self.feed_forward is not None else None
-        ctx.ops.scaled_sum_add(residual, a, self.mixer_scale, f, self.ff_scale)
+        f = self.feed_forward.forward(ctx, h2, residual) if self.feed_forward is not None else None
+        if self.mixer_gate is None and self.ff_gate is None and self.mult == 1.0:
+            ctx.ops.scaled_sum_add(residual, a, self.mixer_scale, f, self.ff_scale)
+            return None
+        if self.mixer_scale is not None or self.ff_scale is not None:
+            raise ValueError("learned column factors beside gates or a multiplier are not built")
+        ctx.ops.gated_sum_add(residual, a, self._gate(ctx, h, self.mixer_gate), self.mixer_gate_bias,
+                              f, self._gate(ctx, h2, self.ff_gate), self.ff_gate_bias, self.mult)
         return None
 
 

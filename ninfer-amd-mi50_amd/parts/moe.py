@@ -34,10 +34,14 @@ class TopKRouter(Part):
     def __init__(self, prefix: str, hidden: int, experts: int, top_k: int, renorm: bool,
                  score: str = "softmax", scale: float = 1.0, choice_bias: bool = False,
                  n_group: int = 0, topk_group: int = 0, group_top: int = 1,
-                 renorm_eps: float = 0.0, leaf: str = "weight"):
+                 renorm_eps: float = 0.0, leaf: str = "weight", weightless: int = 0,
+                 choice_bias_leaf: str = "choice_bias"):
         """`group_top`: a group's score in the group-limited choice is the sum of its group_top
         largest scores (1: its largest). `renorm_eps` is added to the sum of the chosen scores
-        before the division. `leaf`: what follows the prefix in the weight's name."""
+        before the division. `leaf`: what follows the prefix in the weight's name,
+        `choice_bias_leaf` in the bias's. `weightless`: the last so many of the `experts`
+        router outputs stand for experts without weights (they are scored, grouped and chosen
+        like the others; the grouped products pass their rows over)."""
         if top_k > experts:
             raise ValueError(f"top_k ({top_k}) exceeds the number of experts ({experts})")
         if score not in ("softmax", "sigmoid"):
@@ -54,6 +58,9 @@ class TopKRouter(Part):
         # n_group neighbours each) whose best score (+ bias) is largest are candidates
         self.n_group, self.topk_group = int(n_group), int(topk_group)
         self.group_top, self.renorm_eps, self.leaf = int(group_top), float(renorm_eps), leaf
+        self.weightless, self.choice_bias_leaf = int(weightless), choice_bias_leaf
+        if not 0 <= self.weightless < experts:
+            raise ValueError(f"{self.weightless} of {experts} experts without weights")
         if self.n_group > 1 and not 1 <= self.group_top <= experts // max(1, self.n_group):
             raise ValueError(f"group_top ({self.group_top}) must lie in [1, experts per group]")
         if self.n_group > 1 and (experts % self.n_group or not 1 <= self.topk_group <= self.n_group
@@ -66,13 +73,13 @@ class TopKRouter(Part):
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         specs = {self.prefix + self.leaf: TensorSpec((self.experts, self.hidden))}
         if self.has_choice_bias:
-            specs[self.prefix + "choice_bias"] = TensorSpec((self.experts,), role="bias")
+            specs[self.prefix + self.choice_bias_leaf] = TensorSpec((self.experts,), role="bias")
         return specs
 
     def bind(self, w: WeightBinder) -> None:
         self.weight = w.matrix(self.prefix + self.leaf)
         if self.has_choice_bias:
-            self.choice_bias = w.float32(self.prefix + "choice_bias")
+            self.choice_bias = w.float32(self.prefix + self.choice_bias_leaf)
 
     def logits(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
         out = ctx.empty((x.shape[0], self.experts), torch.float32)
@@ -92,7 +99,7 @@ class TopKRouter(Part):
         ctx.ops.moe_route(logits, e, k, self.renorm, r, score=self.score,
                           choice_bias=self.choice_bias, scale=self.scale, n_group=self.n_group,
                           topk_group=self.topk_group, group_top=self.group_top,
-                          renorm_eps=self.renorm_eps)
+                          renorm_eps=self.renorm_eps, weightless=self.weightless)
         return r
 
 
@@ -120,10 +127,13 @@ class RoutedExperts(Part):
     built from the per-expert checkpoint tensors `experts.{e}.*_proj.weight`."""
 
     def __init__(self, prefix: str, hidden: int, inner: int, experts: int, act: str = "silu",
-                 names=("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
+                 names=("gate_proj.weight", "up_proj.weight", "down_proj.weight"),
+                 act_limit: float = 0.0, act_alpha: float = 1.0):
         """`names`: what follows `prefix + str(e) + "."` in the names of expert e's gate, other
-        half and down weights."""
+        half and down weights. `act` 'clamped_swish': g sigmoid(act_alpha g) (u + 1) with g cut
+        at act_limit from above and u to [-act_limit, act_limit]."""
         self.names = tuple(names)
+        self.act_limit, self.act_alpha = float(act_limit), float(act_alpha)
         self.prefix = prefix
         self.hidden = hidden
         self.inner = inner
@@ -159,7 +169,8 @@ class RoutedExperts(Part):
         t, k = routing.ids.shape
         h = ctx.empty((t * k, self.inner))
         ctx.ops.grouped_swiglu(x, self.w_gate_up, routing.offsets, routing.order, k, h,
-                               tiles=routing, act=self.act)
+                               tiles=routing, act=self.act, limit=self.act_limit,
+                               alpha=self.act_alpha)
         return h
 
     def down(self, ctx: StepContext, h: torch.Tensor, routing: "Routing") -> torch.Tensor:
@@ -180,17 +191,25 @@ class SparseMoE(FeedForward):
              "shared": "shared_expert.", "shared_gate": "shared_expert_gate.weight"}
 
     def __init__(self, prefix: str, hidden: int, experts: int, top_k: int, inner: int,
-                 renorm: bool, shared_inner: int = 0, act: str = "silu", router=None, names=None):
+                 renorm: bool, shared_inner: int = 0, act: str = "silu", router=None, names=None,
+                 identity: int = 0, act_limit: float = 0.0, act_alpha: float = 1.0):
         """`router`: further parameters of `TopKRouter` (score, scale, n_group, topk_group,
-        group_top, renorm_eps, choice_bias)."""
+        group_top, renorm_eps, choice_bias, choice_bias_leaf). `identity`: the router has so
+        many outputs beyond the `experts` with weights; the expert of such an output hands its
+        input back (times the weight). `act_limit`, `act_alpha`: see `RoutedExperts`."""
         self.prefix = prefix
         self.hidden = hidden
         n = dict(self.NAMES, **(names or {}))
         self.names = n
-        self.router = TopKRouter(prefix + n["router"], hidden, experts, top_k, renorm,
-                                 leaf=n["router_leaf"], **(router or {}))
+        self.identity = int(identity)
+        if self.identity and shared_inner > 0:
+            raise ValueError("identity experts beside a shared expert are not built")
+        self.router = TopKRouter(prefix + n["router"], hidden, experts + self.identity, top_k,
+                                 renorm, leaf=n["router_leaf"], weightless=self.identity,
+                                 **(router or {}))
         self.experts = RoutedExperts(prefix + n["experts"], hidden, inner, experts, act,
-                                     names=n["expert_leaves"])
+                                     names=n["expert_leaves"], act_limit=act_limit,
+                                     act_alpha=act_alpha)
         self.shared: Optional[SwiGLU] = None
         self.shared_gate: Optional[torch.Tensor] = None
         self.last_ids: Optional[torch.Tensor] = None   # routing of the last step (for statistics)
@@ -226,7 +245,11 @@ class SparseMoE(FeedForward):
             with ctx.ops.together():   # for few rows the logits' block routes the rows itself
                 routing = self.router.route(ctx, self.router.logits(ctx, x))
             self.last_ids = routing.ids
-            return PendingRows(self.experts.run(ctx, x, routing), routing.weights)
+            y = self.experts.run(ctx, x, routing)
+            if self.identity:
+                return PendingRows(y, routing.weights, ids=routing.ids,
+                                   real=self.router.experts - self.identity, rows=x)
+            return PendingRows(y, routing.weights)
         # The shared expert's two products wait for nothing the routed path makes. Many rows:
         # they run on a stream of their own beside the routed path, whose kernels leave part
         # of the device empty in their last round of blocks.

@@ -22,7 +22,8 @@ class TensorSpec:
     """What a part expects of one checkpoint tensor.
 
     role: 'matrix' (kept in the compute dtype), 'gain' (norm weight, read in
-    32-bit, random values 1 + N(0, s)), 'bias' (read in 32-bit).
+    32-bit, random values 1 + N(0, s)), 'bias' (read in 32-bit). A dimension of -1 is one
+    that the checkpoint decides (any size fits; random tensors cannot be made for it).
     """
     shape: Tuple[int, ...]
     role: str = "matrix"
@@ -99,6 +100,9 @@ class RandomSource:
         if name not in self.specs:
             raise WeightError(f"missing tensor in checkpoint: {name}")
         spec = self.specs[name]
+        if any(d < 0 for d in spec.shape):
+            raise WeightError(f"{name}: a size that only a checkpoint decides (shape "
+                              f"{list(spec.shape)}); random weights need it in the configuration")
         key = counter_random.tensor_key(self.seed, name)
         mean = 1.0 if spec.role == "gain" else 0.0
         if torch.device(self.device).type == "cpu":
@@ -124,8 +128,10 @@ def check_tensors(have: Dict[str, Tuple[int, ...]], want: Dict[str, TensorSpec],
     known.update(want)
     missing = sorted(n for n in want if n not in have)
     unexpected = sorted(n for n in have if n not in known)
+    def fits(h, w):
+        return len(h) == len(w) and all(b == -1 or a == b for a, b in zip(h, w))
     wrong = sorted((n, tuple(have[n]), tuple(known[n].shape)) for n in known
-                   if n in have and tuple(have[n]) != tuple(known[n].shape))
+                   if n in have and not fits(tuple(have[n]), tuple(known[n].shape)))
     if not (missing or unexpected or wrong):
         return
     lines = [f"{where}: checkpoint does not match the model"]

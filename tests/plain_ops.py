@@ -128,21 +128,29 @@ class PlainOps:
         out.copy_(r.to(out.dtype))
 
     @staticmethod
+    def _gated(g, u, act, limit=0.0, alpha=1.0):
+        if act == "clamped_swish":
+            g = torch.clamp(g, max=limit)
+            return g / (1 + torch.exp(-alpha * g)) * (torch.clamp(u, -limit, limit) + 1)
+        return PlainOps._act(g, act) * u
+
+    @staticmethod
     def _act(g, act):
         if act == "silu":
             return g / (1 + torch.exp(-g))
         assert act == "gelu_pytorch_tanh", act
         return 0.5 * g * (1 + torch.tanh(math.sqrt(2 / math.pi) * (g + 0.044715 * g ** 3)))
 
-    def swiglu_linear(self, x, w_gate_up, out, act="silu", bias=None):
+    def swiglu_linear(self, x, w_gate_up, out, act="silu", bias=None, limit=0.0, alpha=1.0):
         inner = w_gate_up.shape[0] // 2
         g = _f(x) @ _f(w_gate_up[:inner]).T
         u = _f(x) @ _f(w_gate_up[inner:]).T
         if bias is not None:
             g, u = g + bias[:inner], u + bias[inner:]
-        out.copy_((self._act(g, act) * u).to(out.dtype))
+        out.copy_(self._gated(g, u, act, limit, alpha).to(out.dtype))
 
-    def grouped_swiglu(self, x, w_gate_up, offsets, order, top_k, out, tiles=None, act="silu"):
+    def grouped_swiglu(self, x, w_gate_up, offsets, order, top_k, out, tiles=None, act="silu",
+                       limit=0.0, alpha=1.0):
         e, two_i, _ = w_gate_up.shape
         inner = two_i // 2
         off = offsets.tolist()
@@ -153,7 +161,7 @@ class PlainOps:
             xs = _f(x[rows // top_k])
             gg = xs @ _f(w_gate_up[g, :inner]).T
             uu = xs @ _f(w_gate_up[g, inner:]).T
-            out[off[g]:off[g + 1]] = (self._act(gg, act) * uu).to(out.dtype)
+            out[off[g]:off[g + 1]] = self._gated(gg, uu, act, limit, alpha).to(out.dtype)
 
     def grouped_down(self, h, w_down, offsets, order, out, tiles=None):
         e = w_down.shape[0]
@@ -195,7 +203,7 @@ class PlainOps:
             wts /= wts.sum(-1, keepdim=True) + renorm_eps
         wts *= scale
 
-    def moe_align(self, ids, experts, offsets, order, tiles=None):
+    def moe_align(self, ids, experts, offsets, order, tiles=None, weightless=0):
         flat = ids.reshape(-1).long()
         counts = torch.bincount(flat, minlength=experts)
         offsets[0] = 0
@@ -204,17 +212,17 @@ class PlainOps:
         if tiles is not None and tiles.tiles16 is not None:
             off = offsets.tolist()
             for size, out in ((16, tiles.tiles16), (256, tiles.tiles_big)):
-                lst = [[e, r, off[e + 1], 0] for e in range(experts)
+                lst = [[e, r, off[e + 1], 0] for e in range(experts - weightless)
                        for r in range(off[e], off[e + 1], size)]
                 if lst:
                     out[:len(lst)] = torch.tensor(lst, dtype=torch.int32, device=out.device)
                 tiles.tile_counts[0 if size == 16 else 1] = len(lst)
 
     def moe_route(self, logits, experts, top_k, renorm, r, score="softmax", choice_bias=None,
-                  scale=1.0, n_group=0, topk_group=0, group_top=1, renorm_eps=0.0):
+                  scale=1.0, n_group=0, topk_group=0, group_top=1, renorm_eps=0.0, weightless=0):
         self.router_topk(logits, experts, top_k, renorm, r.ids, r.weights, score, choice_bias,
                          scale, n_group, topk_group, group_top, renorm_eps)
-        self.moe_align(r.ids, experts, r.offsets, r.order, tiles=r)
+        self.moe_align(r.ids, experts, r.offsets, r.order, tiles=r, weightless=weightless)
 
     def paged_attention(self, qkv, k_pool, v_pool, block_table, ctx, n_q, n_kv, head_dim,
                         page_size, window, scale, out, slopes=None):
@@ -270,6 +278,77 @@ class PlainOps:
         else:
             add = _f(f)
         residual += add * (s2 if s2 is not None else 1.0)
+
+    def gated_sum_add(self, residual, a, g1, b1, f, g2, b2, mult=1.0):
+        def gate(g, b):
+            if g is None:
+                return 1.0
+            return torch.sigmoid(_f(g) + (b if b is not None else 0.0))
+        total = torch.zeros_like(residual)
+        if a is not None:
+            total += _f(a) * gate(g1, b1)
+        if f is not None and hasattr(f, "weights"):
+            t, h = residual.shape
+            k = f.weights.shape[1]
+            y = _f(f.y).view(t, k, h)
+            if getattr(f, "ids", None) is not None:
+                back = (f.ids >= f.real)[:, :, None]
+                y = torch.where(back, _f(f.rows)[:, None, :].expand(t, k, h), y)
+            total += (y * f.weights[:, :, None]).sum(1) * gate(g2, b2)
+        elif f is not None:
+            total += _f(f) * gate(g2, b2)
+        residual += mult * total
+
+    def gated_rmsnorm(self, o, gate, weight, eps, out, group=0, gate_act="sigmoid"):
+        t, n = o.shape
+        g = group or n
+        x = o.view(t, n // g, g)
+        x = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * weight
+        z = _f(gate)
+        f = torch.sigmoid(z) * (z if gate_act == "silu" else 1.0)
+        out.copy_((x.reshape(t, n) * f).to(out.dtype))
+
+    def gated_linear_attention(self, qkv, q_off, k_off, v_off, z, heads, dim, vdim, tau, q_scale,
+                               state, ctx, out):
+        starts, slots = ctx.seq_row_start.tolist(), ctx.seq_slots.tolist()
+        alpha = torch.exp(torch.nn.functional.logsigmoid(z) / tau).view(-1, heads, dim)
+        for s, slot in enumerate(slots):
+            st = state[slot, :heads * dim * vdim].view(heads, dim, vdim)
+            for r in range(starts[s], starts[s + 1]):
+                q = _f(qkv[r, q_off:q_off + heads * dim]).view(heads, dim) * q_scale
+                k = _f(qkv[r, k_off:k_off + heads * dim]).view(heads, dim)
+                v = _f(qkv[r, v_off:v_off + heads * vdim]).view(heads, vdim)
+                st.copy_(alpha[r][:, :, None] * st + k[:, :, None] * v[:, None, :])
+                out[r] = torch.einsum("hd,hdv->hv", q, st).reshape(-1)
+
+    def sigmoid_attention(self, qkv, k_pool, v_pool, block_table, ctx, heads, kv_heads, dim, vdim,
+                          page_size, scale, chunk, head_bias, mix, out, write_kv=True):
+        t = qkv.shape[0]
+        nq, nk = heads * dim, kv_heads * dim
+        pos, seq = ctx.positions.tolist(), ctx.row_seq.tolist()
+        if write_kv:
+            for r in range(t):
+                page = int(block_table[seq[r], pos[r] // page_size])
+                assert page >= 0, "write into a page that is not held"
+                k_pool[page, :, pos[r] % page_size] = qkv[r, nq:nq + nk].view(kv_heads, dim)
+                v_pool[page, :, pos[r] % page_size] = qkv[r, nq + nk:].view(kv_heads, vdim)
+        q = _f(qkv[:, :nq]).view(t, heads, dim)
+        per = heads // kv_heads
+        for r in range(t):
+            first = pos[r] // chunk * chunk if chunk else 0
+            js = torch.arange(first, pos[r] + 1)
+            pages = block_table[seq[r], js // page_size].long()
+            assert (pages >= 0).all(), "read of a page that is not held"
+            k = _f(k_pool[pages, :, js % page_size])      # [n, kv_heads, dim]
+            v = _f(v_pool[pages, :, js % page_size])
+            w = torch.stack([k[:, h // per] @ q[r, h] for h in range(heads)]) * scale
+            if head_bias is not None:
+                w = w + head_bias[:, None]
+            w = torch.sigmoid(w)
+            if mix is not None:
+                w = mix @ w
+            for h in range(heads):
+                out[r, h * vdim:(h + 1) * vdim] = (w[h] @ v[:, h // per]).to(out.dtype)
 
     def tanh_cap(self, x, cap):
         x.copy_(cap * torch.tanh(x / cap))
