@@ -29,6 +29,12 @@ runs the same measurement for Sosepel (parallel blocks of differential attention
 sparse feed-forward, a hashed pair embedding, layers that run twice) beside a Qwen2-MoE model of
 the same width, heads and experts with as many layers as the other has layer runs.
 
+    python bench.py --scenario designs --design fopinex [--sizes small,medium] [--only fopinex|sparse]
+
+the same for Fopinex (gated parallel blocks of attention without a softmax or gated linear
+attention and routed experts beside identity experts) beside a Qwen2-MoE model of the same
+width, depth, heads and experts.
+
     python bench.py --scenario long [--model 57b-a14b] [--requests 8] [--prompt 32768] [--new 256]
 
 is another measurement with a JSON line of its own: the scheduler serves
@@ -91,7 +97,7 @@ def main() -> int:
     ap.add_argument("--scenario", default="decode", choices=["decode", "long", "designs"])
     ap.add_argument("--sizes", default="small,medium",
                     help="--scenario designs: which of the layer sizes to run (small, medium)")
-    ap.add_argument("--design", default="getodra", choices=["getodra", "sosepel"],
+    ap.add_argument("--design", default="getodra", choices=["getodra", "sosepel", "fopinex"],
                     help="--scenario designs: the design to run beside the closest model the engine had")
     ap.add_argument("--only", default="", help="--scenario designs: run this one of the two models only")
     ap.add_argument("--requests", type=int, default=8, help="--scenario long: concurrent requests")
@@ -558,21 +564,69 @@ def sparse_config(z: dict) -> dict:
                 use_sliding_window=False)
 
 
+FOPINEX_SIZES = {
+    # width, layers (of every four: attention, attention on the first one's keys and values,
+    # attention, gated linear attention), query and kv heads, sizes of a key and a value, the
+    # chunk of positions a row sees, the recurrence's heads and sizes, experts
+    "small": dict(width=1024, layers=8, heads=8, kv_heads=2, dim=128, vdim=128, chunk=1024,
+                  gla_heads=8, gla_dim=64, gla_vdim=128, rank=32, experts=16, identity=2, top=2,
+                  groups=(3, 2), expert_ff=704, vocab=32000, positions=4096),
+    "medium": dict(width=2048, layers=8, heads=16, kv_heads=4, dim=128, vdim=128, chunk=1024,
+                   gla_heads=16, gla_dim=64, gla_vdim=128, rank=64, experts=32, identity=4, top=4,
+                   groups=(4, 2), expert_ff=1408, vocab=32000, positions=4096),
+}
+
+
+def fopinex_config(z: dict) -> dict:
+    attention = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["vdim"],
+                 "scale": z["dim"] ** -0.5, "mask": {"size": z["chunk"]}}
+    gla = {"heads": z["gla_heads"], "dim": z["gla_dim"], "vdim": z["gla_vdim"], "tau": 16.0,
+           "rank": z["rank"]}
+    moe = {"kind": "moe", "expert": {"ff": z["expert_ff"], "limit": 7.0},
+           "router": {"experts": z["experts"], "identity": z["identity"], "top": z["top"],
+                      "groups": {"count": z["groups"][0], "keep": z["groups"][1]}}}
+    layers = []
+    for i in range(z["layers"]):
+        if i % 4 == 3:
+            layers.append({"type": "gla", "mixer": gla, "mlp": moe})
+        elif i % 4 == 1:
+            layers.append({"type": "attention", "mixer": dict(attention, kv_from=i - 1), "mlp": moe})
+        else:
+            layers.append({"type": "attention", "mixer": attention, "mlp": moe})
+    return {"architecture": "Fopinex", "vocab": z["vocab"], "width": z["width"],
+            "norm": {"eps": 1e-5}, "residual_mult": 0.5, "layers": layers}
+
+
+def sparse_for_fopinex_config(z: dict) -> dict:
+    """The closest model the engine had: Qwen2-MoE blocks (rotary attention with as many query
+    and kv heads of the same size, as many routed experts of the same size, no shared expert)
+    of the same width and depth."""
+    return dict(CONFIG_C, num_hidden_layers=z["layers"], hidden_size=z["width"],
+                num_attention_heads=z["heads"], num_key_value_heads=z["kv_heads"], head_dim=z["dim"],
+                intermediate_size=z["expert_ff"], num_experts=z["experts"],
+                num_experts_per_tok=z["top"], moe_intermediate_size=z["expert_ff"],
+                shared_expert_intermediate_size=0, mlp_only_layers=[], decoder_sparse_step=1,
+                vocab_size=z["vocab"], hidden_act="silu", use_sliding_window=False)
+
+
 def designs_scenario(args) -> int:
     import torch
     from ninfer_amd import Chunk, EngineOptions, random_model
     sosepel = args.design == "sosepel"
 
     gen = torch.Generator().manual_seed(11)
+    fopinex = args.design == "fopinex"
     out = {"metric": "prefill and decode throughput, " + ("Sosepel beside a Qwen2-MoE model" if sosepel
+                     else "Fopinex beside a Qwen2-MoE model" if fopinex
                      else "Getodra beside a dense model") + " of equal size",
            "unit": "tok/s", "n_gpus": 1, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
            "data": "synthetic", "sizes": {}}
     for size in args.sizes.split(","):
-        z = (SOSEPEL_SIZES if sosepel else DESIGN_SIZES)[size]
+        z = (SOSEPEL_SIZES if sosepel else FOPINEX_SIZES if fopinex else DESIGN_SIZES)[size]
         ctx = z["positions"]
         row = {"shape": z}
         pairs = (("sosepel", sosepel_config(z)), ("sparse", sparse_config(z))) if sosepel else \
+            (("fopinex", fopinex_config(z)), ("sparse", sparse_for_fopinex_config(z))) if fopinex else \
             (("getodra", getodra_config(z)), ("dense", dense_config(z)))
         for name, raw in pairs:
             if args.only and name != args.only:
