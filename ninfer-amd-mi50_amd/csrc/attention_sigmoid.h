@@ -20,6 +20,8 @@ struct SigAttnArgs {
   const int* seq_row_start; // [S + 1]
   const float* head_bias;   // [Hq] added to the scaled score, or null
   const float* mix;         // [Hq, Hq] row a: the weights of head a's mixture, or null
+  float* workspace;         // partial outputs of key ranges cut into parts, or null
+  int64_t workspace_floats;
   int q_stride;
   int bt_stride;
   int T;
@@ -39,8 +41,11 @@ struct SigAttnArgs {
 };
 
 int sigmoid_attention_plain(const SigAttnArgs& a, hipStream_t stream);
+// the matrix-core kernel: row tiles of all heads, the visible keys cut into n_splits parts
+// whose partial outputs (`part`: n_splits x T x Hq x vdim 32-bit numbers, null with one
+// part) a second kernel adds up
 bool sigmoid_attention_tiles_takes(const SigAttnArgs& a);
-// (the requests before `first_seq` are left out: their single rows run on the plain kernel)
-int sigmoid_attention_tiles(const SigAttnArgs& a, int first_seq, hipStream_t stream);
+int sigmoid_attention_tiles_splits(const SigAttnArgs& a);
+int sigmoid_attention_tiles(const SigAttnArgs& a, float* part, int n_splits, hipStream_t stream);
 
 }  // namespace ninfer

@@ -165,8 +165,24 @@ extern "C" int ninfer_sigmoid_kv_write(const SigAttnArgs* a, hipStream_t stream)
   return 0;
 }
 
+// 32-bit scratch the call needs (0: none): the partial outputs of the matrix-core kernel.
+extern "C" long long ninfer_sigmoid_attention_workspace_floats(const SigAttnArgs* a) {
+  if (sigmoid_check(*a, "sigmoid_attention")) return 0;
+  if (a->force_plain || !sigmoid_attention_tiles_takes(*a)) return 0;
+  const int n = sigmoid_attention_tiles_splits(*a);
+  return n > 1 ? (long long)n * a->T * a->Hq * a->vdim : 0;
+}
+
 extern "C" int ninfer_sigmoid_attention(const SigAttnArgs* a, hipStream_t stream) {
   int rc = sigmoid_check(*a, "sigmoid_attention");
   if (rc) return rc;
+  NINFER_REQUIRE(a->out && a->qkv && a->kpool && a->vpool, "sigmoid_attention: null tensors");
+  if (!a->force_plain && sigmoid_attention_tiles_takes(*a)) {
+    const int n = sigmoid_attention_tiles_splits(*a);
+    if (n > 1)
+      NINFER_REQUIRE(a->workspace && a->workspace_floats >= (int64_t)n * a->T * a->Hq * a->vdim,
+                     "sigmoid_attention: the workspace is too small for %d parts", n);
+    return sigmoid_attention_tiles(*a, a->workspace, n, stream);
+  }
   return sigmoid_attention_plain(*a, stream);
 }

@@ -133,7 +133,8 @@ class _SigAttnArgs(ctypes.Structure):
                 ("out", ctypes.c_void_p), ("block_table", ctypes.c_void_p),
                 ("positions", ctypes.c_void_p), ("row_seq", ctypes.c_void_p),
                 ("seq_row_start", ctypes.c_void_p), ("head_bias", ctypes.c_void_p),
-                ("mix", ctypes.c_void_p),
+                ("mix", ctypes.c_void_p), ("workspace", ctypes.c_void_p),
+                ("workspace_floats", ctypes.c_int64),
                 ("q_stride", ctypes.c_int), ("bt_stride", ctypes.c_int), ("T", ctypes.c_int),
                 ("S", ctypes.c_int), ("Hq", ctypes.c_int), ("Hkv", ctypes.c_int),
                 ("dim", ctypes.c_int), ("vdim", ctypes.c_int), ("page_size", ctypes.c_int),
@@ -255,6 +256,7 @@ class HipOps:
         self.lib.ninfer_sample_few_places.restype = ctypes.c_longlong
         self.lib.ninfer_latent_attention_workspace_floats.restype = ctypes.c_longlong
         self.lib.ninfer_diff_attention_workspace_floats.restype = ctypes.c_longlong
+        self.lib.ninfer_sigmoid_attention_workspace_floats.restype = ctypes.c_longlong
         self.force_generic = False  # tests: run the plain kernels whatever the shape
         self._device_index = None   # the one GPU's index, asked for at the first launch
         self._held = None           # products held back inside `together()`
@@ -1393,6 +1395,10 @@ class HipOps:
         a.single_rows = int(getattr(ctx, "single_rows", 0))
         if write_kv:
             self._ok(self.lib.ninfer_sigmoid_kv_write(ctypes.byref(a), self._stream()))
+        need = int(self.lib.ninfer_sigmoid_attention_workspace_floats(ctypes.byref(a)))
+        if need:   # the visible keys cut into parts: partial outputs, added up by a second kernel
+            ws = self._workspace(need, qkv.device)
+            a.workspace, a.workspace_floats = ws.data_ptr(), ws.numel()
         self._ok(self.lib.ninfer_sigmoid_attention(ctypes.byref(a), self._stream()))
 
     # ---- sampling -------------------------------------------------------------------

@@ -133,22 +133,26 @@ def expert(w, prefix: str, limit: float, h: torch.Tensor) -> torch.Tensor:
     return lin(w, prefix + "down", g * torch.sigmoid(1.702 * g) * (u + 1))
 
 
-def moe(w, prefix: str, mlp: dict, h: torch.Tensor, margins: Optional[List[float]] = None):
+def moe(w, prefix: str, mlp: dict, h: torch.Tensor, margins: Optional[List[torch.Tensor]] = None):
+    """`margins` receives, per call, how clear every row's routing was (see `route`)."""
     ids, wts, margin = route(w, prefix, mlp, h)
     if margins is not None:
-        margins.append(float(margin.min()))
+        margins.append(margin)
     real = mlp["router"]["experts"]
     out = torch.zeros_like(h)
-    for t in range(h.shape[0]):
-        for e, p in zip(ids[t].tolist(), wts[t]):
-            if e >= real:                      # an identity expert hands its input back
-                out[t] += p * h[t]
-            else:
-                out[t] += p * expert(w, f"{prefix}e{e}.", mlp["expert"]["limit"], h[t:t + 1])[0]
+    for e in range(real + mlp["router"].get("identity", 0)):
+        share = torch.where(ids == e, wts, torch.zeros((), dtype=D)).sum(-1)      # [n]
+        rows = share.nonzero().flatten()
+        if rows.numel() == 0:
+            continue
+        x = h[rows]
+        # an identity expert hands its input back
+        y = x if e >= real else expert(w, f"{prefix}e{e}.", mlp["expert"]["limit"], x)
+        out[rows] += share[rows, None] * y
     return out
 
 
-def forward(cfg: dict, w: Dict[str, torch.Tensor], tokens, margins: Optional[List[float]] = None):
+def forward(cfg: dict, w: Dict[str, torch.Tensor], tokens, margins: Optional[List[torch.Tensor]] = None):
     """(logits [n, vocab], the residual stream after every layer [L, n, width]) of one whole
     sequence from position 0."""
     eps = cfg["norm"]["eps"]
