@@ -10,18 +10,21 @@
 // request may be cut into steps anywhere and every row sees exactly the sums it would see in
 // one piece.
 //
-// One wave owns 16 value columns of one (request, head) and walks the request's rows of the
-// step in order. Lane (part, col) keeps S[d][col] for the DPL key channels d = part DPL ..
-// in registers, updates them and forms its part of o_t[col]; the four parts are added by two
-// lane exchanges. q, k and the decay of a row are staged in LDS (the wave's lanes each fetch
-// a channel, a row ahead of the one being computed). The order of every sum depends on dim
-// alone.
+// A block of four waves owns 64 value columns of one (request, head) and walks the request's
+// rows of the step in order; a wave owns 16 of the columns. Lane (part, col) keeps S[d][col]
+// for the DPL key channels d = part DPL .. in registers, updates them and forms its part of
+// o_t[col]; the four parts are added by two lane exchanges. q, k and the decay of a row are
+// staged in LDS by the block's threads, a channel each (two buffers, one barrier a row); the
+// rows come from global memory eight at a time, one batch ahead of the one being computed, so
+// that the loads' latency is paid once per batch. The order of every sum depends on dim alone.
 #include "common.h"
 
 namespace ninfer {
 
 constexpr int kGlaCols = 16;    // value columns per wave
 constexpr int kGlaParts = 4;    // parts of the key channels, one per 16 lanes
+constexpr int kGlaWaves = 4;    // waves per block
+constexpr int kGlaBatch = 8;    // rows fetched at a time
 
 __device__ __forceinline__ float log_sigmoid(float z) {
   return fminf(z, 0.f) - log1pf(expf(-fabsf(z)));
@@ -41,12 +44,13 @@ struct GlaArgs {
 };
 
 template <typename T, int DPL>
-__global__ __launch_bounds__(64) void gla_seq_kernel(GlaArgs a) {
+__global__ __launch_bounds__(64 * kGlaWaves) void gla_seq_kernel(GlaArgs a) {
   constexpr int DIM = DPL * kGlaParts;            // channels held (>= dim; the rest stay 0)
-  constexpr int PER_LANE = (DIM + 63) / 64;       // channels a lane fetches
+  static_assert(DIM <= 64 * kGlaWaves, "a thread stages one channel");
   __shared__ __attribute__((aligned(16))) float q_s[2][DIM], k_s[2][DIM], a_s[2][DIM];
-  const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const int col = blockIdx.z * kGlaCols + (lane & (kGlaCols - 1)), part = lane / kGlaCols;
+  const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = (blockIdx.z * kGlaWaves + wave) * kGlaCols + (lane & (kGlaCols - 1));
+  const int part = lane / kGlaCols;
   const bool has_col = col < a.vdim;
   const int r0 = a.seq_row_start[s], n = a.seq_row_start[s + 1] - r0;
   const int dim = a.dim, vdim = a.vdim;
@@ -58,47 +62,57 @@ __global__ __launch_bounds__(64) void gla_seq_kernel(GlaArgs a) {
     const int d = part * DPL + i;
     S[i] = has_col && d < dim ? st[(int64_t)d * vdim + col] : 0.f;
   }
-  // the row a lane fetches ahead: q, k and the decay's logit of its channels, and v of its column
-  float fq[PER_LANE], fk[PER_LANE], fz[PER_LANE], fv = 0.f;
-  auto fetch = [&](int row) {
-    const T* r = (const T*)a.qkv + (int64_t)row * a.stride;
-    const float* zr = a.z + ((int64_t)row * a.H + h) * dim;
+  // the batch of rows a thread fetches ahead: q, k and the decay's logit of its channel (thread
+  // tid looks after channel tid), and v of its column
+  const bool stages = tid < DIM, in_dim = tid < dim;
+  float fq[kGlaBatch], fk[kGlaBatch], fz[kGlaBatch], fv[kGlaBatch];
+  auto fetch = [&](int first) {
 #pragma unroll
-    for (int i = 0; i < PER_LANE; ++i) {
-      const int d = lane + 64 * i;
-      const bool in = d < dim;
-      fq[i] = in ? to_f32(r[a.q_off + h * dim + d]) : 0.f;
-      fk[i] = in ? to_f32(r[a.k_off + h * dim + d]) : 0.f;
-      fz[i] = in ? zr[d] : 0.f;
+    for (int j = 0; j < kGlaBatch; ++j) {
+      const int row = r0 + min(first + j, n - 1);   // (rows beyond the last are fetched again, not used)
+      const T* r = (const T*)a.qkv + (int64_t)row * a.stride;
+      fq[j] = in_dim ? to_f32(r[a.q_off + h * dim + tid]) : 0.f;
+      fk[j] = in_dim ? to_f32(r[a.k_off + h * dim + tid]) : 0.f;
+      fz[j] = in_dim ? a.z[((int64_t)row * a.H + h) * dim + tid] : 0.f;
+      fv[j] = has_col ? to_f32(r[a.v_off + h * vdim + col]) : 0.f;
     }
-    fv = has_col ? to_f32(r[a.v_off + h * vdim + col]) : 0.f;
   };
-  if (n > 0) fetch(r0);
-  for (int i = 0; i < n; ++i) {
-    const int b = i & 1;
+  if (n > 0) fetch(0);
+  for (int base = 0; base < n; base += kGlaBatch) {
+    float cq[kGlaBatch], ck[kGlaBatch], ca[kGlaBatch], cv[kGlaBatch];
 #pragma unroll
-    for (int j = 0; j < PER_LANE; ++j) {
-      const int d = lane + 64 * j;
-      if (d < DIM) {
-        q_s[b][d] = fq[j] * a.q_scale;
-        k_s[b][d] = fk[j];
-        a_s[b][d] = d < dim ? expf(log_sigmoid(fz[j]) * a.inv_tau) : 1.f;
+    for (int j = 0; j < kGlaBatch; ++j) {
+      cq[j] = fq[j] * a.q_scale;
+      ck[j] = fk[j];
+      ca[j] = in_dim ? expf(log_sigmoid(fz[j]) * a.inv_tau) : 1.f;
+      cv[j] = fv[j];
+    }
+    if (base + kGlaBatch < n) fetch(base + kGlaBatch);
+#pragma unroll
+    for (int j = 0; j < kGlaBatch; ++j) {
+      if (base + j >= n) break;
+      const int b = j & 1;
+      if (stages) {
+        q_s[b][tid] = cq[j];
+        k_s[b][tid] = ck[j];
+        a_s[b][tid] = ca[j];
       }
-    }
-    const float v_t = fv;
-    __syncthreads();   // the row is in LDS; the other buffer's readers are done
-    if (i + 1 < n) fetch(r0 + i + 1);
-    float o = 0.f;
+      // (a barrier that waits for LDS traffic only: the batch on its way and the outputs' stores
+      // stay in flight)
+      lds_barrier();   // the row is in LDS; the other buffer's readers are done
+      const float v_t = cv[j];
+      float o = 0.f;
 #pragma unroll
-    for (int j = 0; j < DPL; ++j) {
-      const int d = part * DPL + j;
-      const float sn = fmaf(a_s[b][d], S[j], k_s[b][d] * v_t);
-      S[j] = sn;
-      o = fmaf(sn, q_s[b][d], o);
+      for (int i = 0; i < DPL; ++i) {
+        const int d = part * DPL + i;
+        const float sn = fmaf(a_s[b][d], S[i], k_s[b][d] * v_t);
+        S[i] = sn;
+        o = fmaf(sn, q_s[b][d], o);
+      }
+      o += __shfl_xor(o, 16, 64);
+      o += __shfl_xor(o, 32, 64);
+      if (part == 0 && has_col) a.out[((int64_t)(r0 + base + j) * a.H + h) * vdim + col] = o;
     }
-    o += __shfl_xor(o, 16, 64);
-    o += __shfl_xor(o, 32, 64);
-    if (part == 0 && has_col) a.out[((int64_t)(r0 + i) * a.H + h) * vdim + col] = o;
   }
 #pragma unroll
   for (int i = 0; i < DPL; ++i) {
@@ -134,11 +148,12 @@ extern "C" int ninfer_gated_linear_attention(const void* qkv, int stride, int q_
   a.seq_row_start = seq_row_start, a.seq_slots = seq_slots, a.state_stride = state_stride;
   a.stride = stride, a.q_off = q_off, a.k_off = k_off, a.v_off = v_off;
   a.H = H, a.dim = dim, a.vdim = vdim, a.inv_tau = 1.f / tau, a.q_scale = q_scale;
-  const dim3 grid(S, H, (vdim + kGlaCols - 1) / kGlaCols);
+  const int cols = kGlaCols * kGlaWaves;
+  const dim3 grid(S, H, (vdim + cols - 1) / cols);
 #define NINFER_GLA(DPL)                                                             \
   do {                                                                              \
-    if (dtype == kF32) gla_seq_kernel<float, DPL><<<grid, 64, 0, stream>>>(a);      \
-    else gla_seq_kernel<bf16, DPL><<<grid, 64, 0, stream>>>(a);                     \
+    if (dtype == kF32) gla_seq_kernel<float, DPL><<<grid, 64 * kGlaWaves, 0, stream>>>(a);      \
+    else gla_seq_kernel<bf16, DPL><<<grid, 64 * kGlaWaves, 0, stream>>>(a);                     \
   } while (0)
   if (dim <= 16) NINFER_GLA(4);
   else if (dim <= 32) NINFER_GLA(8);
