@@ -279,6 +279,7 @@ class HipOps:
         # (65: a decode step of up to 64 rows takes the same kernels run eagerly and captured)
         self.beside_heavy_min_rows = 65
         self.beside_heavy_bytes = 256 << 20
+        self.gla_chunk_min_rows = 8         # the same for gated linear attention
         self.lightning_chunk_min_rows = 8   # a step's longest portion from which lightning attention runs in chunks
         self.library_min_rows = 32  # dense bf16 products with more rows go to the library
         self.rows_kernel_max = 64   # ... unless the kernel for 33 to 64 rows takes them
@@ -1324,13 +1325,25 @@ class HipOps:
         self._ok(self.lib.ninfer_gated_sum_add(ctypes.byref(p), self._stream()))
         del keep
 
+    def gla_work_floats(self, qkv_dtype, ctx, heads, dim):
+        """The size of the workspace with which `gated_linear_attention` runs this step in
+        chunks, per row; 0 if the step runs token by token."""
+        if qkv_dtype != torch.bfloat16 or ctx.max_qlen < self.gla_chunk_min_rows or self.force_generic \
+                or dim > 128 or dim % 4:
+            return 0
+        return 3 * heads * dim + 16 * heads
+
     def gated_linear_attention(self, qkv, q_off, k_off, v_off, z, heads, dim, vdim, tau, q_scale,
-                               state, ctx, out):
+                               state, ctx, out, work=None):
         """Linear attention with a decay per key channel and token over the rows of each
         request: S <- diag(alpha) S + k v^T, out = S^T (q q_scale) with alpha =
         sigmoid(z)^(1 / tau), q, k at the columns q_off, k_off (heads x dim) and v at v_off
         (heads x vdim) of `qkv`; z: [T, heads * dim] 32-bit. `state` ([slots, >= heads * dim *
-        vdim] 32-bit view) holds every request's S between steps. out: [T, heads * vdim] 32-bit."""
+        vdim] 32-bit view) holds every request's S between steps. out: [T, heads * vdim] 32-bit.
+        `work` ([T, gla_work_floats(..)] 32-bit, or None): with it a bfloat16 step that brings
+        prompt portions runs in chunks of 16 rows on the matrix cores (the sums of a chunk are
+        ordered otherwise than token by token, so the 32-bit path, whose logits do not depend
+        on the cut to the bit, stays on the token-by-token kernel)."""
         _dev(qkv, "qkv", dims=2)
         _dev(z, "z", torch.float32, 2)
         _dev(out, "out", torch.float32, 2)
@@ -1343,6 +1356,22 @@ class HipOps:
         _need(state.is_cuda and state.dtype == torch.float32 and state.dim() == 2
               and state.stride(1) == 1 and state.shape[1] >= heads * dim * vdim,
               "gated_linear_attention: the state must be 32-bit rows of heads * dim * vdim numbers")
+        if work is not None and self.gla_work_floats(qkv.dtype, ctx, heads, dim):
+            _dev(work, "work", torch.float32, 2)
+            _need(work.is_contiguous() and work.shape[0] == t
+                  and work.shape[1] >= 3 * heads * dim + 16 * heads,
+                  "gated_linear_attention: the workspace is too small")
+            rc = self.lib.ninfer_gated_linear_attention_chunks(
+                ctypes.c_void_p(qkv.data_ptr()), qkv.shape[1], q_off, k_off, v_off,
+                ctypes.c_void_p(z.data_ptr()), ctypes.c_float(tau), ctypes.c_float(q_scale),
+                ctypes.c_void_p(state.data_ptr()), ctypes.c_longlong(state.stride(0)),
+                ctypes.c_void_p(out.data_ptr()), ctypes.c_void_p(ctx.seq_row_start.data_ptr()),
+                ctypes.c_void_p(ctx.seq_slots.data_ptr()), ctypes.c_void_p(work.data_ptr()),
+                t, ctx.S, heads, dim, vdim, _DT[qkv.dtype], self._stream())
+            if rc == 0:
+                return
+            if rc < 0:
+                self._ok(rc)
         self._ok(self.lib.ninfer_gated_linear_attention(
             ctypes.c_void_p(qkv.data_ptr()), qkv.shape[1], q_off, k_off, v_off,
             ctypes.c_void_p(z.data_ptr()), ctypes.c_float(tau), ctypes.c_float(q_scale),

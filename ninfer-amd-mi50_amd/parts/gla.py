@@ -88,8 +88,11 @@ class GatedLinearAttention(Mixer):
         z = ctx.empty((ctx.T, qk), torch.float32)     # the decay's logits, 32-bit from here on
         ops.linear(low, self.w_a2, z, bias=self.b_a2)
         o = ctx.empty((ctx.T, v), torch.float32)
+        # (a step with prompt portions runs in chunks, which keep their scaled rows here)
+        wf = ops.gla_work_floats(proj.dtype, ctx, self.heads, self.dim)
+        work = ctx.empty((ctx.T, wf), torch.float32) if wf else None
         ops.gated_linear_attention(proj, 0, qk, 2 * qk, z, self.heads, self.dim, self.vdim,
-                                   self.tau, self.q_scale, call.state, ctx, o)
+                                   self.tau, self.q_scale, call.state, ctx, o, work=work)
         gated = ctx.empty((ctx.T, v))
         ops.gated_rmsnorm(o, proj[:, 2 * qk + v:], self.norm_w, self.eps, gated, group=self.vdim,
                           gate_act="silu")

@@ -308,8 +308,11 @@ class PlainOps:
         f = torch.sigmoid(z) * (z if gate_act == "silu" else 1.0)
         out.copy_((x.reshape(t, n) * f).to(out.dtype))
 
+    def gla_work_floats(self, qkv_dtype, ctx, heads, dim):
+        return 0
+
     def gated_linear_attention(self, qkv, q_off, k_off, v_off, z, heads, dim, vdim, tau, q_scale,
-                               state, ctx, out):
+                               state, ctx, out, work=None):
         starts, slots = ctx.seq_row_start.tolist(), ctx.seq_slots.tolist()
         alpha = torch.exp(torch.nn.functional.logsigmoid(z) / tau).view(-1, heads, dim)
         for s, slot in enumerate(slots):

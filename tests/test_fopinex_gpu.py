@@ -322,12 +322,16 @@ def _gla_plain(rows, z, heads, dim, vdim, tau, q_scale):
     return out
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype,chunks", [(torch.float32, False), (torch.bfloat16, False),
+                                          (torch.bfloat16, True)])
 @pytest.mark.parametrize("heads,dim,vdim,tau", [(3, 10, 12, 5.0), (2, 64, 64, 16.0), (1, 128, 32, 1.0),
-                                                (4, 16, 100, 2.0), (2, 200, 24, 8.0), (5, 33, 17, 0.5)])
-def test_gated_linear_attention_in_portions(ops, dtype, heads, dim, vdim, tau):
+                                                (4, 16, 100, 2.0), (2, 200, 24, 8.0), (5, 33, 17, 0.5),
+                                                (3, 12, 20, 5.0), (2, 40, 130, 0.5), (1, 4, 1, 1.0)])
+def test_gated_linear_attention_in_portions(ops, dtype, chunks, heads, dim, vdim, tau):
     """Three requests in slots 2, 0 and 3 of a wider state tensor, cut into portions down to
-    two rows and single rows, with logits that drive some decays to 0 and some to 1."""
+    two rows and single rows, with logits that drive some decays to 0 and some to 1; token by
+    token, and with the workspace that lets steps with longer portions run in chunks (sizes
+    that the chunks refuse fall back by themselves)."""
     lens = [150, 9, 77]
     rows, z = _gla_rows(heads, dim, vdim, lens, dim * vdim, dtype)
     z[0][:, :3] = 40.0          # decay 1: a channel that never forgets
@@ -344,8 +348,10 @@ def test_gated_linear_attention_in_portions(ops, dtype, heads, dim, vdim, tau):
         x = torch.cat([rows[r][s:s + n] for r, s, n in zip(who, starts, counts)]).to(DEV)
         zz = torch.cat([z[r][s:s + n] for r, s, n in zip(who, starts, counts)]).to(DEV)
         out = torch.empty(ctx.T, heads * vdim, device=DEV)
+        wf = ops.gla_work_floats(dtype, ctx, heads, dim) if chunks else 0
+        work = torch.full((ctx.T, wf), float("nan"), device=DEV) if wf else None
         ops.gated_linear_attention(x, 5, 5 + heads * dim, 5 + 2 * heads * dim, zz, heads, dim, vdim, tau,
-                                   dim ** -0.5, view, ctx, out)
+                                   dim ** -0.5, view, ctx, out, work=work)
         o = 0
         for r, s, n in zip(who, starts, counts):
             got[r][s:s + n] = out[o:o + n].cpu()
