@@ -82,7 +82,7 @@ def main() -> int:
     ap.add_argument("--no-check", action="store_true",
                     help="skip the comparison of replayed with eager decode steps (untimed)")
     ap.add_argument("--prefill-tokens", type=int, default=2048,
-                    help="length of the timed prefill (the contract's figure is at 2,048)")
+                    help="length of the timed prefill (the headline figure is at 2,048)")
     ap.add_argument("--graph", dest="graph", action="store_true", default=True,
                     help="decode steps replayed from a captured HIP graph (the default)")
     ap.add_argument("--no-graph", dest="graph", action="store_false",
@@ -565,8 +565,8 @@ def sparse_config(z: dict) -> dict:
 
 
 FOPINEX_SIZES = {
-    # width, layers (of every four: attention, attention on the first one's keys and values,
-    # attention, gated linear attention), query and kv heads, sizes of a key and a value, the
+    # width, layers (of every four: attention, gated linear attention, attention on the first
+    # one's keys and values, attention), query and kv heads, sizes of a key and a value, the
     # chunk of positions a row sees, the recurrence's heads and sizes, experts
     "small": dict(width=1024, layers=8, heads=8, kv_heads=2, dim=128, vdim=128, chunk=1024,
                   gla_heads=8, gla_dim=64, gla_vdim=128, rank=32, experts=16, identity=2, top=2,
@@ -580,21 +580,21 @@ FOPINEX_SIZES = {
 def fopinex_config(z: dict) -> dict:
     attention = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["vdim"],
                  "scale": z["dim"] ** -0.5, "mask": {"size": z["chunk"]}}
-    gla = {"heads": z["gla_heads"], "dim": z["gla_dim"], "vdim": z["gla_vdim"], "tau": 16.0,
+    gla = {"heads": z["gla_heads"], "dim": z["gla_dim"], "vdim": z["gla_vdim"], "tau": 8.0,
            "rank": z["rank"]}
     moe = {"kind": "moe", "expert": {"ff": z["expert_ff"], "limit": 7.0},
            "router": {"experts": z["experts"], "identity": z["identity"], "top": z["top"],
                       "groups": {"count": z["groups"][0], "keep": z["groups"][1]}}}
     layers = []
     for i in range(z["layers"]):
-        if i % 4 == 3:
+        if i % 4 == 1:
             layers.append({"type": "gla", "mixer": gla, "mlp": moe})
-        elif i % 4 == 1:
-            layers.append({"type": "attention", "mixer": dict(attention, kv_from=i - 1), "mlp": moe})
+        elif i % 4 == 2:
+            layers.append({"type": "attention", "mixer": dict(attention, kv_from=i - 2), "mlp": moe})
         else:
             layers.append({"type": "attention", "mixer": attention, "mlp": moe})
     return {"architecture": "Fopinex", "vocab": z["vocab"], "width": z["width"],
-            "norm": {"eps": 1e-5}, "residual_mult": 0.5, "layers": layers}
+            "norm": {"eps": 1e-6}, "residual_mult": 0.7, "layers": layers}
 
 
 def sparse_for_fopinex_config(z: dict) -> dict:
