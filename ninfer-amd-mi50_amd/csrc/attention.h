@@ -35,13 +35,18 @@ struct AttnArgs {
                             // 0 .. single_rows - 1 (0 when the caller does not sort them)
   const float* slopes;      // [Hq] or null: head h's scores get slopes[h] * (key position - row's
                             // position) added before the softmax (a distance-based position bias)
+  int Dv;                   // numbers of a value head: vpool is [pages, Hkv, page_size, Dv] and out
+                            // [T, Hq*Dv] (0: the same as D)
+  int sink;                 // != 0: the softmax's denominator has one more term, exp(0), that
+                            // belongs to no key (a sink with score 0 and no value)
 };
 
 int attention_check(const AttnArgs& a);
 int attention_generic(const void* q, int q_stride, const void* kpool, const void* vpool,
                       const int* block_table, int bt_stride, const int* positions,
                       const int* row_seq, void* out, int T, int Hq, int Hkv, int D, int page_size,
-                      int window, float scale, const float* slopes, int dtype, hipStream_t stream);
+                      int window, float scale, const float* slopes, int dtype, int Dv, int sink,
+                      hipStream_t stream);
 
 int64_t attention_decode_workspace_floats(int T, int Hq, int D, int max_kv_len);
 bool attention_decode_takes(const AttnArgs& a);
@@ -51,5 +56,11 @@ bool attention_decode_heads_takes(const AttnArgs& a);
 int attention_decode_heads(const AttnArgs& a, int chunk, int n_chunks, hipStream_t stream);
 bool attention_prefill_takes(const AttnArgs& a);
 int attention_prefill(const AttnArgs& a, hipStream_t stream);
+// keys of D and values of Dv numbers (multiples of 8 up to 256), a window or none, a sink or
+// none: row tiles on the matrix cores; single rows with the heads of a kv head as the tile's rows
+bool attention_tiles_takes(const AttnArgs& a);
+int attention_tiles(const AttnArgs& a, int first_seq, hipStream_t stream);
+bool attention_tiles_heads_takes(const AttnArgs& a);
+int attention_tiles_heads(const AttnArgs& a, hipStream_t stream);
 
 }  // namespace ninfer

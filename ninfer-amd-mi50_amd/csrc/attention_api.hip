@@ -20,6 +20,7 @@ int attention_check(const AttnArgs& args) {
                  a->dtype);
   NINFER_REQUIRE(a->q_stride >= a->Hq * a->D, "paged_attention: row stride %d < %d", a->q_stride,
                  a->Hq * a->D);
+  NINFER_REQUIRE(a->Dv >= 0, "paged_attention: value size %d is negative", a->Dv);
   NINFER_REQUIRE(a->max_qlen >= 1 && a->max_kv_len >= 1, "paged_attention: bad size hints");
   NINFER_REQUIRE(a->single_rows >= 0 && a->single_rows <= a->S && a->single_rows <= a->T,
                  "paged_attention: %d single rows of %d requests", a->single_rows, a->S);
@@ -54,9 +55,25 @@ extern "C" int ninfer_paged_attention(const AttnArgs* a, int force_generic, hipS
     return attention_prefill(p, stream);
   }
   if (!force_generic && attention_prefill_takes(*a)) return attention_prefill(*a, stream);
+  // keys and values of sizes of their own, a sink: row tiles of any such shape on the matrix
+  // cores; single rows (which come first) with the heads of a kv head as a tile's rows
+  if (!force_generic && attention_tiles_takes(*a)) {
+    const int n = a->max_qlen == 1 ? a->S : a->single_rows;
+    if (n > 0 && attention_tiles_heads_takes(*a)) {
+      AttnArgs d = *a;
+      d.T = n;
+      d.S = n;
+      d.max_qlen = 1;
+      if (int rc = attention_tiles_heads(d, stream)) return rc;
+      if (n == a->S) return 0;
+      return attention_tiles(*a, n, stream);
+    }
+    return attention_tiles(*a, 0, stream);
+  }
   return attention_generic(a->q, a->q_stride, a->kpool, a->vpool, a->block_table, a->bt_stride,
                            a->positions, a->row_seq, a->out, a->T, a->Hq, a->Hkv, a->D,
-                           a->page_size, a->window, a->scale, a->slopes, a->dtype, stream);
+                           a->page_size, a->window, a->scale, a->slopes, a->dtype, a->Dv, a->sink,
+                           stream);
 }
 
 // 32-bit floats of workspace the split-KV decode kernel needs for this shape.

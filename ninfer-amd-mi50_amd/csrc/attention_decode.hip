@@ -278,7 +278,8 @@ bool attention_decode_takes(const AttnArgs& a) {
   int d = a.D;
   bool d_ok = d == 16 || d == 32 || d == 64 || d == 128 || d == 256;
   bool ps_ok = (a.page_size & (a.page_size - 1)) == 0;
-  return a.dtype == kBF16 && d_ok && ps_ok && a.q_stride % 8 == 0 && a.workspace != nullptr;
+  return a.dtype == kBF16 && d_ok && ps_ok && a.q_stride % 8 == 0 && a.workspace != nullptr &&
+         (a.Dv == 0 || a.Dv == a.D) && !a.sink;
 }
 
 template <int LPK, int CHUNK>

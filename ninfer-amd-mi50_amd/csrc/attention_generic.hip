@@ -9,7 +9,9 @@
 // the request was cut into steps or what else is in the batch. Query head h
 // reads kv head h / (Hq / Hkv) (reference src/ops/attention.hip:27-28).
 // Scores, softmax and the value sum are 32-bit. This is the kernel of the true
-// 32-bit path and of head sizes the MFMA kernels refuse.
+// 32-bit path and of head sizes the MFMA kernels refuse. Values may have another size than
+// keys (Dv), and the softmax may have a sink: one more term exp(0) in its denominator that
+// belongs to no key, so that the weights of a row add up to less than one.
 #include "common.h"
 
 namespace ninfer {
@@ -22,11 +24,11 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
     const T* __restrict__ vpool, const int* __restrict__ block_table, int bt_stride,
     const int* __restrict__ positions, const int* __restrict__ row_seq, T* __restrict__ out,
     int Hq, int Hkv, int D, int page_size, int window, float scale,
-    const float* __restrict__ slopes) {
+    const float* __restrict__ slopes, int Dv, int sink) {
   extern __shared__ float smem[];
   float* q_s = smem;                 // [D]
   float* p_s = smem + D;             // [64]
-  int64_t* off_s = (int64_t*)(p_s + 64);  // [64] element offset of each key's row
+  int64_t* off_s = (int64_t*)(p_s + 64);  // [64] page's slot (page * Hkv + g) * page_size + slot of each key
 
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int g = h / (Hq / Hkv);
@@ -39,7 +41,8 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
   for (int d = lane; d < D; d += 64) q_s[d] = to_f32(qr[d]);
   __syncthreads();
 
-  float m = -INFINITY, l = 0.f;
+  // (a sink is a key with score 0 and no value: the running maximum starts at 0, the sum at 1)
+  float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
   float acc[kMaxDPerLane];
 #pragma unroll
   for (int i = 0; i < kMaxDPerLane; ++i) acc[i] = 0.f;
@@ -51,8 +54,8 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
     int64_t off = 0;
     if (valid) {
       int page = bt[j / page_size];
-      off = (((int64_t)page * Hkv + g) * page_size + (j % page_size)) * D;
-      const T* kr = kpool + off;
+      off = ((int64_t)page * Hkv + g) * page_size + (j % page_size);
+      const T* kr = kpool + off * D;
       float dot = 0.f;
       for (int d = 0; d < D; ++d) dot = fmaf(q_s[d], to_f32(kr[d]), dot);
       s = fmaf(slope, (float)(j - pos), dot * scale);
@@ -70,39 +73,41 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
 #pragma unroll
     for (int i = 0; i < kMaxDPerLane; ++i) {
       int d = lane + i * 64;
-      if (d < D) {
+      if (d < Dv) {
         float a = acc[i] * alpha;
-        for (int jj = first; jj < n_keys; ++jj) a = fmaf(p_s[jj], to_f32(vpool[off_s[jj] + d]), a);
+        for (int jj = first; jj < n_keys; ++jj) a = fmaf(p_s[jj], to_f32(vpool[off_s[jj] * Dv + d]), a);
         acc[i] = a;
       }
     }
     __syncthreads();
   }
-  T* orow = out + ((int64_t)t * Hq + h) * D;
+  T* orow = out + ((int64_t)t * Hq + h) * Dv;
   float inv = 1.f / l;
 #pragma unroll
   for (int i = 0; i < kMaxDPerLane; ++i) {
     int d = lane + i * 64;
-    if (d < D) orow[d] = from_f32<T>(acc[i] * inv);
+    if (d < Dv) orow[d] = from_f32<T>(acc[i] * inv);
   }
 }
 
 int attention_generic(const void* q, int q_stride, const void* kpool, const void* vpool,
                       const int* block_table, int bt_stride, const int* positions,
                       const int* row_seq, void* out, int T, int Hq, int Hkv, int D, int page_size,
-                      int window, float scale, const float* slopes, int dtype, hipStream_t stream) {
-  NINFER_REQUIRE(D <= 64 * kMaxDPerLane, "paged_attention: head size %d exceeds %d", D,
-                 64 * kMaxDPerLane);
+                      int window, float scale, const float* slopes, int dtype, int Dv, int sink,
+                      hipStream_t stream) {
+  if (Dv <= 0) Dv = D;
+  NINFER_REQUIRE(D <= 64 * kMaxDPerLane && Dv <= 64 * kMaxDPerLane,
+                 "paged_attention: head sizes %d, %d exceed %d", D, Dv, 64 * kMaxDPerLane);
   dim3 grid(T, Hq);
   size_t lds = (D + 64) * sizeof(float) + 64 * sizeof(int64_t);
   if (dtype == kF32)
     paged_attention_generic_kernel<float><<<grid, 64, lds, stream>>>(
         (const float*)q, q_stride, (const float*)kpool, (const float*)vpool, block_table, bt_stride,
-        positions, row_seq, (float*)out, Hq, Hkv, D, page_size, window, scale, slopes);
+        positions, row_seq, (float*)out, Hq, Hkv, D, page_size, window, scale, slopes, Dv, sink);
   else
     paged_attention_generic_kernel<bf16><<<grid, 64, lds, stream>>>(
         (const bf16*)q, q_stride, (const bf16*)kpool, (const bf16*)vpool, block_table, bt_stride,
-        positions, row_seq, (bf16*)out, Hq, Hkv, D, page_size, window, scale, slopes);
+        positions, row_seq, (bf16*)out, Hq, Hkv, D, page_size, window, scale, slopes, Dv, sink);
   NINFER_LAUNCH_CHECK();
   return 0;
 }

@@ -26,8 +26,8 @@
 //                    into chunks over several blocks whose partial sums a second kernel
 //                    merges (steps of few rows would otherwise leave most of the GPU idle).
 //
-// The rotation turns pair (i, i + n/2) of the first n = rot_n numbers of the rotated part by
-// pos * freq[i]; cosine and sine are multiplied by `magnitude` (1 without a scaled table).
+// The rotation turns pair (i, i + n/2), or with `interleaved` pair (2i, 2i + 1), of the first
+// n = rot_n numbers of the rotated part by pos * freq[i]; cosine and sine are multiplied by `magnitude` (1 without a scaled table).
 // Norm, angles, scores, softmax and the value sum are 32-bit.
 #include "common.h"
 
@@ -70,6 +70,7 @@ struct LatentArgs {
   float eps;
   float magnitude;
   float scale;
+  int interleaved;          // pair i of the turning numbers is (2i, 2i + 1) instead of (i, i + rot_n / 2)
 };
 
 __device__ __forceinline__ void turn_pair(float u, float v, float c, float s, float* a, float* b) {
@@ -109,10 +110,11 @@ __global__ void latent_kv_write_kernel(LatentArgs a) {
     for (int i = threadIdx.x; i < a.rd; i += blockDim.x) {
       float v = to_f32(kr[i]);
       if (i < a.rot_n) {
-        const int p = i < half ? i : i - half;
+        const int p = a.interleaved ? i >> 1 : i < half ? i : i - half;
+        const int i1 = a.interleaved ? 2 * p : p, i2 = a.interleaved ? 2 * p + 1 : p + half;
         float x, y;
-        turn_pair(to_f32(kr[p]), to_f32(kr[p + half]), trig[p], trig[half + p], &x, &y);
-        v = i < half ? x : y;
+        turn_pair(to_f32(kr[i1]), to_f32(kr[i2]), trig[p], trig[half + p], &x, &y);
+        v = i == i1 ? x : y;
       }
       dst[a.R + i] = from_f32<T>(v);
     }
@@ -123,10 +125,11 @@ __global__ void latent_kv_write_kernel(LatentArgs a) {
     const T* qr = (const T*)a.q + ((int64_t)t * a.Hq + h) * qd + a.dim;
     float v = to_f32(qr[i]);
     if (i < a.rot_n) {
-      const int p = i < half ? i : i - half;
+      const int p = a.interleaved ? i >> 1 : i < half ? i : i - half;
+      const int i1 = a.interleaved ? 2 * p : p, i2 = a.interleaved ? 2 * p + 1 : p + half;
       float x, y;
-      turn_pair(to_f32(qr[p]), to_f32(qr[p + half]), trig[p], trig[half + p], &x, &y);
-      v = i < half ? x : y;
+      turn_pair(to_f32(qr[i1]), to_f32(qr[i2]), trig[p], trig[half + p], &x, &y);
+      v = i == i1 ? x : y;
     }
     a.q_abs[((int64_t)t * a.Hq + h) * Dk + a.R + i] = v;
   }

@@ -535,7 +535,7 @@ bool attention_decode_heads_takes(const AttnArgs& a) {
   const int group = a.Hq / a.Hkv;
   return a.dtype == kBF16 && (a.D == 64 || a.D == 128) && a.q_stride % 8 == 0 &&
          prefill_page_ok(a) && group >= 3 && group <= 32 && a.workspace != nullptr &&
-         a.row_seq != nullptr;
+         a.row_seq != nullptr && (a.Dv == 0 || a.Dv == a.D) && !a.sink;
 }
 
 // Pass 1 of split-context decoding for grouped heads; the caller merges the chunks.
@@ -551,7 +551,7 @@ int attention_decode_heads(const AttnArgs& a, int chunk, int n_chunks, hipStream
 
 bool attention_prefill_takes(const AttnArgs& a) {
   return a.dtype == kBF16 && (a.D == 64 || a.D == 128) && a.q_stride % 8 == 0 &&
-         prefill_page_ok(a) && a.seq_row_start != nullptr;
+         prefill_page_ok(a) && a.seq_row_start != nullptr && (a.Dv == 0 || a.Dv == a.D) && !a.sink;
 }
 
 // Row tiles of PQ rows that the launch enumerates (one more per request than whole tiles:

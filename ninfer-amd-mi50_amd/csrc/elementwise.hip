@@ -81,7 +81,7 @@ __device__ __forceinline__ void store_vec(bf16* p, const float* f) {
 template <typename T, int VEC>
 __global__ void rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delta, MoeSum ms,
                                const float* __restrict__ gain, T* __restrict__ out,
-                               const int* __restrict__ rows, int H, float eps) {
+                               const int* __restrict__ rows, int H, float eps, int center) {
   constexpr int G = kNormPerThread / VEC;   // groups per thread
   __shared__ float red[16];
   int64_t r_out = blockIdx.x;
@@ -148,11 +148,27 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delt
       }
     }
   }
+  // with `center` the row's mean is taken off first (a layer norm without a bias): the mean of
+  // the squared deviations stands where the mean of the squares stood
+  float mean = 0.f;
+  if (center) {
+    float sum = 0.f;
+#pragma unroll
+    for (int c = 0; c < G; ++c)
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) sum += vals[c][e];   // (places beyond H hold zeros)
+    mean = block_sum(sum, red) / (float)H;
+  }
   float acc = 0.f;
 #pragma unroll
-  for (int c = 0; c < G; ++c)
+  for (int c = 0; c < G; ++c) {
+    const bool in = VEC * (threadIdx.x + c * blockDim.x) < H;
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) acc += vals[c][e] * vals[c][e];
+    for (int e = 0; e < VEC; ++e) {
+      const float dv = in ? vals[c][e] - mean : 0.f;
+      acc += dv * dv;
+    }
+  }
   float total = block_sum(acc, red);
   float inv = rsqrtf(total / (float)H + eps);
   const bool write_back = !rows && (dr || ms.y);
@@ -164,7 +180,7 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delt
       float gv[VEC], o[VEC];
       load_vec<VEC>(gain + i, gv);
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) o[e] = vals[c][e] * inv * gv[e];
+      for (int e = 0; e < VEC; ++e) o[e] = (vals[c][e] - mean) * inv * gv[e];
       store_vec<VEC>(orow + i, o);
     }
   }
@@ -436,7 +452,7 @@ extern "C" int ninfer_rmsnorm(float* x, const void* delta, const float* gain, vo
                               const int* rows, int n_rows, int H, float eps, int dtype,
                               const void* moe_y, const float* moe_w, const void* moe_shared,
                               const float* moe_gate, int moe_gate_stride, int moe_k,
-                              hipStream_t stream) {
+                              int center, hipStream_t stream) {
   NINFER_REQUIRE(n_rows > 0 && H > 0, "rmsnorm: rows=%d H=%d must be positive", n_rows, H);
   NINFER_REQUIRE(dtype == kF32 || dtype == kBF16, "rmsnorm: unknown dtype %d", dtype);
   NINFER_REQUIRE(H <= 1024 * kNormPerThread, "rmsnorm: width %d exceeds %d", H,
@@ -455,17 +471,17 @@ extern "C" int ninfer_rmsnorm(float* x, const void* delta, const float* gain, vo
   if (dtype == kF32) {
     if (vec)
       rmsnorm_kernel<float, 4><<<n_rows, block, 0, stream>>>(x, (const float*)delta, ms, gain,
-                                                            (float*)out, rows, H, eps);
+                                                            (float*)out, rows, H, eps, center);
     else
       rmsnorm_kernel<float, 1><<<n_rows, block, 0, stream>>>(x, (const float*)delta, ms, gain,
-                                                            (float*)out, rows, H, eps);
+                                                            (float*)out, rows, H, eps, center);
   } else {
     if (vec)
       rmsnorm_kernel<bf16, 4><<<n_rows, block, 0, stream>>>(x, (const bf16*)delta, ms, gain,
-                                                           (bf16*)out, rows, H, eps);
+                                                           (bf16*)out, rows, H, eps, center);
     else
       rmsnorm_kernel<bf16, 1><<<n_rows, block, 0, stream>>>(x, (const bf16*)delta, ms, gain,
-                                                           (bf16*)out, rows, H, eps);
+                                                           (bf16*)out, rows, H, eps, center);
   }
   NINFER_LAUNCH_CHECK();
   return 0;

@@ -4,7 +4,9 @@
 //                  rows of each request, channel by channel, added to its input. The last
 //                  taps - 1 inputs of a request are per-request state (32-bit), so a request
 //                  may be cut into steps anywhere; before a request's start they are zero.
-//   norm_add       x += y rsqrt(mean(y^2) + eps) g, g one number or one per channel.
+//   norm_add       x += y rsqrt(mean(y^2) + eps) g, g one number or one per channel; optionally
+//                  with the row's mean taken off first (a layer norm), and with y a weighted
+//                  sum of rows.
 //   gated_rmsnorm  out = o rsqrt(mean(o^2) + eps) w sigmoid(g) (or w g sigmoid(g)), the norm
 //                  over the whole row or over every group of columns (a head's) by itself.
 //
@@ -65,23 +67,49 @@ __global__ void short_conv_state_kernel(const float* __restrict__ x, float* __re
   }
 }
 
+// x += norm(y) g with norm(y) = y rsqrt(mean(y^2) + eps), or with `center` the layer norm
+// (y - mean) rsqrt(mean((y - mean)^2) + eps). y is a row of `y`, or with `w` the weighted sum of
+// k rows, y_r = sum_j w[r, j] y[r k + j] (a sparse feed-forward's chosen experts), formed in
+// 32-bit in the order of j. A thread keeps its (at most 8) numbers of the row in registers.
+constexpr int kNormAddPerThread = 8;
 template <typename T>
 __global__ void norm_add_kernel(float* __restrict__ x, const T* __restrict__ y,
-                                const float* __restrict__ gain, int gain_n, int H, float eps) {
+                                const float* __restrict__ w, int k,
+                                const float* __restrict__ gain, int gain_n, int H, float eps,
+                                int center) {
   __shared__ float red[16];
   const int64_t r = blockIdx.x;
-  const T* yr = y + r * H;
+  float vals[kNormAddPerThread];
+  float sum = 0.f;
+#pragma unroll
+  for (int c = 0; c < kNormAddPerThread; ++c) {
+    const int i = threadIdx.x + c * blockDim.x;
+    float v = 0.f;
+    if (i < H) {
+      if (w) {
+        for (int j = 0; j < k; ++j) v = fmaf(w[r * k + j], to_f32(y[(r * k + j) * H + i]), v);
+      } else {
+        v = to_f32(y[r * H + i]);
+      }
+    }
+    vals[c] = v;
+    sum += v;
+  }
+  const float mean = center ? block_sum(sum, red) / (float)H : 0.f;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) {
-    const float v = to_f32(yr[i]);
-    ss = fmaf(v, v, ss);
+#pragma unroll
+  for (int c = 0; c < kNormAddPerThread; ++c) {
+    const int i = threadIdx.x + c * blockDim.x;
+    const float d = i < H ? vals[c] - mean : 0.f;
+    ss = fmaf(d, d, ss);
   }
   ss = block_sum(ss, red);
   const float inv = 1.f / sqrtf(ss / (float)H + eps);
   float* xr = x + r * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) {
-    const float g = gain[gain_n == 1 ? 0 : i];
-    xr[i] += to_f32(yr[i]) * inv * g;
+#pragma unroll
+  for (int c = 0; c < kNormAddPerThread; ++c) {
+    const int i = threadIdx.x + c * blockDim.x;
+    if (i < H) xr[i] += (vals[c] - mean) * inv * gain[gain_n == 1 ? 0 : i];
   }
 }
 
@@ -164,15 +192,19 @@ extern "C" int ninfer_short_conv(const float* x, const float* w, float* state,
 }
 
 extern "C" int ninfer_norm_add(float* x, const void* y, const float* gain, int gain_n, int T, int H,
-                               float eps, int dtype, hipStream_t stream) {
+                               float eps, int dtype, int center, const float* w, int k,
+                               hipStream_t stream) {
   NINFER_REQUIRE(T > 0 && H > 0, "norm_add: T=%d H=%d must be positive", T, H);
   NINFER_REQUIRE(gain_n == 1 || gain_n == H, "norm_add: %d gains for %d channels", gain_n, H);
   NINFER_REQUIRE(dtype == kF32 || dtype == kBF16, "norm_add: unknown dtype %d", dtype);
+  NINFER_REQUIRE(H <= 1024 * kNormAddPerThread, "norm_add: width %d exceeds %d", H,
+                 1024 * kNormAddPerThread);
+  NINFER_REQUIRE(!w || k > 0, "norm_add: a weighted sum of %d rows", k);
   const int block = H >= 1024 ? 1024 : (H + 63) / 64 * 64;
   if (dtype == kF32)
-    norm_add_kernel<float><<<T, block, 0, stream>>>(x, (const float*)y, gain, gain_n, H, eps);
+    norm_add_kernel<float><<<T, block, 0, stream>>>(x, (const float*)y, w, k, gain, gain_n, H, eps, center);
   else
-    norm_add_kernel<bf16><<<T, block, 0, stream>>>(x, (const bf16*)y, gain, gain_n, H, eps);
+    norm_add_kernel<bf16><<<T, block, 0, stream>>>(x, (const bf16*)y, w, k, gain, gain_n, H, eps, center);
   NINFER_LAUNCH_CHECK();
   return 0;
 }

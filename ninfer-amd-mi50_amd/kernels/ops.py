@@ -80,7 +80,22 @@ class _AttnArgs(ctypes.Structure):
                 ("D", ctypes.c_int), ("page_size", ctypes.c_int), ("window", ctypes.c_int),
                 ("scale", ctypes.c_float), ("dtype", ctypes.c_int), ("max_qlen", ctypes.c_int),
                 ("max_kv_len", ctypes.c_int), ("single_rows", ctypes.c_int),
-                ("slopes", ctypes.c_void_p)]
+                ("slopes", ctypes.c_void_p), ("Dv", ctypes.c_int), ("sink", ctypes.c_int)]
+
+
+class _QkvConvArgs(ctypes.Structure):
+    _fields_ = [("u", ctypes.c_void_p), ("w", ctypes.c_void_p), ("state", ctypes.c_void_p),
+                ("state_stride", ctypes.c_int64), ("q_out", ctypes.c_void_p),
+                ("kpool", ctypes.c_void_p), ("vpool", ctypes.c_void_p),
+                ("block_table", ctypes.c_void_p), ("positions", ctypes.c_void_p),
+                ("row_seq", ctypes.c_void_p), ("seq_row_start", ctypes.c_void_p),
+                ("seq_slots", ctypes.c_void_p), ("q_gain", ctypes.c_void_p),
+                ("k_gain", ctypes.c_void_p), ("inv_freq", ctypes.c_void_p),
+                ("bt_stride", ctypes.c_int), ("T", ctypes.c_int), ("S", ctypes.c_int),
+                ("Hq", ctypes.c_int), ("Hkv", ctypes.c_int), ("dim", ctypes.c_int),
+                ("vdim", ctypes.c_int), ("taps", ctypes.c_int), ("rot_dim", ctypes.c_int),
+                ("interleaved", ctypes.c_int), ("page_size", ctypes.c_int),
+                ("dtype", ctypes.c_int), ("eps", ctypes.c_float)]
 
 
 class _QkvRopeArgs(ctypes.Structure):
@@ -109,7 +124,8 @@ class _LatentArgs(ctypes.Structure):
                 ("Hq", ctypes.c_int), ("dim", ctypes.c_int), ("R", ctypes.c_int),
                 ("rd", ctypes.c_int), ("rot_n", ctypes.c_int), ("page_size", ctypes.c_int),
                 ("window", ctypes.c_int), ("write_kv", ctypes.c_int), ("dtype", ctypes.c_int),
-                ("eps", ctypes.c_float), ("magnitude", ctypes.c_float), ("scale", ctypes.c_float)]
+                ("eps", ctypes.c_float), ("magnitude", ctypes.c_float), ("scale", ctypes.c_float),
+                ("interleaved", ctypes.c_int)]
 
 
 class _DiffAttnArgs(ctypes.Structure):
@@ -404,9 +420,11 @@ class HipOps:
             ctypes.c_void_p(_ptr(pos_table)), 0 if pos_table is None else pos_table.shape[0],
             self._stream()))
 
-    def rmsnorm(self, x, gain, eps, out, delta=None, rows=None, rows_sum=None):
+    def rmsnorm(self, x, gain, eps, out, delta=None, rows=None, rows_sum=None, center=False):
         """out = norm(x [+ delta] [+ rows_sum]); `rows_sum` is a weighted sum of
-        rows (an object with y, weights, shared, gate) added on the fly."""
+        rows (an object with y, weights, shared, gate) added on the fly. norm(v) =
+        v rsqrt(mean(v^2) + eps) gain, or with `center` the layer norm without a bias,
+        (v - mean(v)) rsqrt(mean((v - mean(v))^2) + eps) gain."""
         _dev(x, "x", torch.float32, 2)
         _dev(gain, "gain", torch.float32, 1)
         _dev(out, "out", dims=2)
@@ -430,7 +448,7 @@ class HipOps:
             ctypes.c_void_p(gain.data_ptr()), ctypes.c_void_p(out.data_ptr()),
             ctypes.c_void_p(_ptr(rows)), out.shape[0], h, ctypes.c_float(eps), _DT[out.dtype],
             ctypes.c_void_p(my), ctypes.c_void_p(mw), ctypes.c_void_p(msh), ctypes.c_void_p(mg),
-            mgs, mk, self._stream()))
+            mgs, mk, 1 if center else 0, self._stream()))
 
     @staticmethod
     def _check_rows_sum(rs, t, h, dtype):
@@ -874,22 +892,27 @@ class HipOps:
 
     # ---- attention ------------------------------------------------------------------
     def paged_attention(self, qkv, k_pool, v_pool, block_table, ctx, n_q, n_kv, head_dim,
-                        page_size, window, scale, out, plan_only=False, slopes=None):
+                        page_size, window, scale, out, plan_only=False, slopes=None, vdim=None,
+                        sink=False):
         """Attention of the rows' query heads (the first n_q * head_dim columns
         of `qkv`) over their requests' cached keys and values. `slopes` [n_q] (32-bit): head
         h's scores get slopes[h] * (key's position - row's position) added before the softmax
         (a distance-based position bias; negative distances, so a positive slope favours near
-        keys). `plan_only`: launch
+        keys). `vdim`: numbers of a value head when they differ from a key head's (`v_pool` and
+        `out` are that wide). `sink`: the softmax's denominator has one more term, exp(0), that
+        belongs to no key. `plan_only`: launch
         nothing and say how a step of single-token rows of this shape would run
         (which split-context kernel, keys per chunk, chunks)."""
+        vdim = head_dim if vdim is None else int(vdim)
         _dev(qkv, "qkv", dims=2)
         _dev(k_pool, "k_pool", qkv.dtype, 4)
         _dev(v_pool, "v_pool", qkv.dtype, 4)
         _dev(out, "out", qkv.dtype, 2)
         _dev(block_table, "block_table", torch.int32, 2)
         t = qkv.shape[0]
-        _need(out.shape == (t, n_q * head_dim), "paged_attention: out has the wrong shape")
-        _need(k_pool.shape == v_pool.shape and k_pool.shape[1:] == (n_kv, page_size, head_dim),
+        _need(out.shape == (t, n_q * vdim), "paged_attention: out has the wrong shape")
+        _need(k_pool.shape[0] == v_pool.shape[0] and k_pool.shape[1:] == (n_kv, page_size, head_dim)
+              and v_pool.shape[1:] == (n_kv, page_size, vdim),
               "paged_attention: pools do not fit the head layout")
         _need(block_table.shape[0] == ctx.S, "paged_attention: block table rows != requests")
         _need(ctx.positions.shape[0] == t, "paged_attention: positions size")
@@ -919,7 +942,7 @@ class HipOps:
             ctx.seq_row_start.data_ptr(), ctx.seq_qlen.data_ptr(), ctx.seq_pos0.data_ptr(),
             ws, ws_floats, qkv.shape[1], block_table.shape[1], t, ctx.S, n_q, n_kv, head_dim, page_size,
             int(window or 0), float(scale), _DT[qkv.dtype], ctx.max_qlen, ctx.max_kv_len, single,
-            _ptr(slopes))
+            _ptr(slopes), vdim, 1 if sink else 0)
         if plan_only:
             kernel, chunk, n_chunks = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
             self._ok(self.lib.ninfer_attention_decode_plan(
@@ -929,6 +952,64 @@ class HipOps:
                     "chunks": n_chunks.value}
         self._ok(self.lib.ninfer_paged_attention(ctypes.byref(args),
                                                  1 if self.force_generic else 0, self._stream()))
+
+    def qkv_conv(self, u, w_conv, state, ctx, q_out, heads, kv_heads, dim, vdim, k_pool, v_pool,
+                 block_table, page_size, q_norm=None, k_norm=None, norm_eps=0.0, inv_freq=None,
+                 rot_dim=0, interleaved=False):
+        """Projected rows u [T, heads * dim + kv_heads * (dim + vdim)] on their way to attention:
+        a causal convolution over time per channel (`w_conv` [channels, taps], None: none; the
+        taps - 1 projected rows before a step's first row come from `state` [slots, >= (taps - 1)
+        * channels] 32-bit, which is moved on), then query and key heads normed over their `dim`
+        numbers (gains `q_norm`, `k_norm` [dim], None: no norm) and turned by their position
+        (`inv_freq`, `rot_dim`, pairing as in `rope_kv_write`); queries to `q_out` [T, heads *
+        dim], keys and values to the requests' pages of `k_pool` [pages, kv_heads, page_size,
+        dim] and `v_pool` [.., vdim]. kv_heads 0: the rows hold queries only."""
+        _dev(u, "u", dims=2)
+        _dev(q_out, "q_out", u.dtype, 2)
+        t = ctx.T
+        channels = heads * dim + kv_heads * (dim + vdim)
+        _need(u.dtype in _DT and u.shape == (t, channels) and q_out.shape == (t, heads * dim),
+              f"qkv_conv: rows of {tuple(u.shape)} for {channels} channels")
+        a = _QkvConvArgs()
+        a.u, a.q_out = u.data_ptr(), q_out.data_ptr()
+        taps = 0
+        if w_conv is not None:
+            _dev(w_conv, "w_conv", torch.float32, 2)
+            taps = w_conv.shape[1]
+            _need(w_conv.shape[0] == channels and taps >= 1, "qkv_conv: one row of taps per channel")
+            a.w = w_conv.data_ptr()
+        if taps > 1:
+            _need(state is not None and state.is_cuda and state.dtype == torch.float32
+                  and state.dim() == 2 and state.stride(1) == 1
+                  and state.shape[1] >= (taps - 1) * channels,
+                  "qkv_conv: the state must be 32-bit rows of at least (taps - 1) * channels numbers")
+            a.state, a.state_stride = state.data_ptr(), state.stride(0)
+        if kv_heads:
+            _dev(k_pool, "k_pool", u.dtype, 4)
+            _dev(v_pool, "v_pool", u.dtype, 4)
+            _dev(block_table, "block_table", torch.int32, 2)
+            _need(k_pool.shape[0] == v_pool.shape[0]
+                  and k_pool.shape[1:] == (kv_heads, page_size, dim)
+                  and v_pool.shape[1:] == (kv_heads, page_size, vdim) and block_table.shape[0] == ctx.S,
+                  "qkv_conv: pools or block table do not fit the head layout")
+            a.kpool, a.vpool, a.block_table = k_pool.data_ptr(), v_pool.data_ptr(), block_table.data_ptr()
+            a.bt_stride = block_table.shape[1]
+        for g, name in ((q_norm, "q_norm"), (k_norm, "k_norm")):
+            if g is not None:
+                _dev(g, name, torch.float32, 1)
+                _need(g.shape[0] == dim, f"qkv_conv: {name} has one gain per number of a head")
+        _need(kv_heads == 0 or (q_norm is None) == (k_norm is None), "qkv_conv: both heads' norms or neither")
+        a.q_gain, a.k_gain = _ptr(q_norm), _ptr(k_norm)
+        if rot_dim:
+            _dev(inv_freq, "inv_freq", torch.float32, 1)
+            _need(inv_freq.shape[0] == rot_dim // 2 and rot_dim <= dim, "qkv_conv: table size != rot_dim / 2")
+            a.inv_freq = inv_freq.data_ptr()
+        a.positions, a.row_seq = ctx.positions.data_ptr(), ctx.row_seq.data_ptr()
+        a.seq_row_start, a.seq_slots = ctx.seq_row_start.data_ptr(), ctx.seq_slots.data_ptr()
+        a.T, a.S, a.Hq, a.Hkv, a.dim, a.vdim, a.taps = t, ctx.S, heads, kv_heads, dim, vdim, taps
+        a.rot_dim, a.interleaved, a.page_size = rot_dim, 1 if interleaved else 0, page_size
+        a.dtype, a.eps = _DT[u.dtype], norm_eps
+        self._ok(self.lib.ninfer_qkv_conv(ctypes.byref(a), self._stream()))
 
     # ---- sublayers with the norm on their output -----------------------------------
     def short_conv(self, x, w, state, ctx, out):
@@ -959,17 +1040,29 @@ class HipOps:
             ctypes.c_void_p(ctx.seq_row_start.data_ptr()), ctypes.c_void_p(ctx.seq_slots.data_ptr()),
             t, ctx.S, h, taps, 1 if ctx.max_qlen == 1 else 0, _DT[out.dtype], self._stream()))
 
-    def norm_add(self, residual, y, gain, eps):
-        """residual += y rsqrt(mean(y^2) + eps) gain; gain holds one number or one per column."""
+    def norm_add(self, residual, y, gain, eps, center=False, weights=None):
+        """residual += y rsqrt(mean(y^2) + eps) gain; gain holds one number or one per column.
+        `center`: the layer norm instead, (y - mean(y)) rsqrt(mean((y - mean(y))^2) + eps) gain.
+        `weights` [T, k] (32-bit): y holds T * k rows and stands for the rows
+        sum_j weights[t, j] y[t * k + j], formed in 32-bit (a sparse feed-forward's output)."""
         _dev(residual, "residual", torch.float32, 2)
         _dev(y, "y", dims=2)
         _dev(gain, "gain", torch.float32, 1)
-        _need(y.shape == residual.shape and y.dtype in _DT, "norm_add: y does not fit the residual")
+        k = 0
+        if weights is not None:
+            _dev(weights, "weights", torch.float32, 2)
+            k = weights.shape[1]
+            _need(weights.shape[0] == residual.shape[0] and y.shape == (residual.shape[0] * k,
+                  residual.shape[1]), "norm_add: the weighted rows do not fit the residual")
+        else:
+            _need(y.shape == residual.shape, "norm_add: y does not fit the residual")
+        _need(y.dtype in _DT, "norm_add: y's dtype")
         _need(gain.shape[0] in (1, y.shape[1]), "norm_add: one gain, or one per column")
         self._ok(self.lib.ninfer_norm_add(
             ctypes.c_void_p(residual.data_ptr()), ctypes.c_void_p(y.data_ptr()),
-            ctypes.c_void_p(gain.data_ptr()), gain.shape[0], y.shape[0], y.shape[1],
-            ctypes.c_float(eps), _DT[y.dtype], self._stream()))
+            ctypes.c_void_p(gain.data_ptr()), gain.shape[0], residual.shape[0], y.shape[1],
+            ctypes.c_float(eps), _DT[y.dtype], 1 if center else 0,
+            ctypes.c_void_p(_ptr(weights)), k, self._stream()))
 
     def gated_rmsnorm(self, o, gate, weight, eps, out, group=0, gate_act="sigmoid"):
         """out = o rsqrt(mean(o^2) + eps) weight sigmoid(gate), the mean over the whole row, or
@@ -1049,13 +1142,15 @@ class HipOps:
         return a
 
     def latent_kv_write(self, dkv, q, q_abs, pool, block_table, ctx, heads, dim, rank, rot_dim,
-                        norm_w, eps, freq, rot_n, magnitude, page_size, write_kv=True):
+                        norm_w, eps, freq, rot_n, magnitude, page_size, write_kv=True,
+                        interleaved=False):
         """Per row: the first `rank` columns of `dkv` normed (x rsqrt(mean(x^2) + eps) norm_w)
         and the next `rot_dim`, turned by the row's position, go to the request's page of
         `pool` [pages, page_size, rank + rot_dim]; the rotated part of every head of `q`
         ([T, heads * (dim + rot_dim)]) is turned and written behind the first `rank` numbers of
         the head's row of `q_abs` [T, heads, rank + rot_dim] (32-bit). Pair (i, i + rot_n / 2)
-        of the first rot_n rotated numbers turns by pos * freq[i]; cos and sin times `magnitude`."""
+        (with `interleaved`: pair (2i, 2i + 1)) of the first rot_n rotated numbers turns by
+        pos * freq[i]; cos and sin times `magnitude`."""
         _need(dkv.is_cuda and dkv.dim() == 2 and dkv.stride(1) == 1 and dkv.shape[1] >= rank + rot_dim,
               "latent_kv_write: dkv must be rows of at least rank + rot_dim columns")
         _dev(q, "q", dkv.dtype, 2)
@@ -1074,6 +1169,7 @@ class HipOps:
         a.dkv, a.q, a.q_abs, a.norm_w = dkv.data_ptr(), q.data_ptr(), q_abs.data_ptr(), norm_w.data_ptr()
         a.dkv_stride = dkv.stride(0) if t > 1 else max(dkv.shape[1], dkv.stride(0))
         a.eps, a.magnitude, a.scale, a.write_kv = eps, magnitude, 1.0, 1 if write_kv else 0
+        a.interleaved = 1 if interleaved else 0
         self._ok(self.lib.ninfer_latent_kv_write(ctypes.byref(a), self._stream()))
 
     def latent_attention(self, q_abs, pool, block_table, ctx, heads, rank, rot_dim, page_size,

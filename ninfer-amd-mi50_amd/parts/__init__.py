@@ -1,7 +1,7 @@
 from .attention import Attention
 from .base import (Block, CacheNeed, CacheView, CallInfo, FeedForward, Mixer, Norm, Part,
                    PendingRows, PoolSpec, PositionEncoding, StepContext, WeightBinder, settle)
-from .block import OutputNormBlock, ParallelBlock, PreNormBlock
+from .block import OutputNormBlock, ParallelBlock, PreNormBlock, SandwichBlock
 from .diff_attention import DifferentialAttention
 from .embedding import LMHead, TokenEmbedding
 from .gla import GatedLinearAttention
@@ -9,7 +9,7 @@ from .latent_attention import LatentAttention
 from .lightning import LightningAttention
 from .mlp import MLP, SwiGLU
 from .moe import RoutedExperts, Routing, SoftmaxTopKRouter, SparseMoE, TopKRouter
-from .norm import OutputRMSNorm, RMSNorm
+from .norm import LayerNorm, OutputLayerNorm, OutputRMSNorm, RMSNorm
 from .rotary import NoPosition, Rotary
 from .reentry import StreamReentry
 from .short_conv import ShortConv
@@ -21,4 +21,4 @@ __all__ = ["Attention", "Block", "CacheNeed", "CacheView", "CallInfo", "FeedForw
            "SparseMoE", "RMSNorm", "NoPosition", "Rotary", "OutputNormBlock", "OutputRMSNorm",
            "LatentAttention", "LightningAttention", "ShortConv", "ParallelBlock",
            "DifferentialAttention", "MLP", "StreamReentry", "GatedLinearAttention",
-           "SigmoidAttention"]
+           "SigmoidAttention", "SandwichBlock", "LayerNorm", "OutputLayerNorm"]

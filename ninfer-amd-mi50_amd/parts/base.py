@@ -51,11 +51,12 @@ class CacheNeed:
 
     @staticmethod
     def keys_values(kv_heads: int, head_dim: int, window: Optional[int] = None,
-                    page_size: Optional[int] = None) -> "CacheNeed":
-        """Keys and values of `kv_heads` heads of `head_dim`: pools 'k' and 'v',
-        each [pages, kv_heads, page_size, head_dim]."""
+                    page_size: Optional[int] = None, vdim: Optional[int] = None) -> "CacheNeed":
+        """Keys and values of `kv_heads` heads of `head_dim` (values: `vdim`, when given):
+        pools 'k' [pages, kv_heads, page_size, head_dim] and 'v' [.., vdim]."""
         return CacheNeed((PoolSpec("k", (kv_heads,), (head_dim,)),
-                          PoolSpec("v", (kv_heads,), (head_dim,))), window, page_size)
+                          PoolSpec("v", (kv_heads,), (head_dim if vdim is None else vdim,))),
+                         window, page_size)
 
 
 @dataclass

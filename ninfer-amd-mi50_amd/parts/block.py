@@ -98,6 +98,40 @@ class OutputNormBlock(Block):
 register_part("block", "output_norm", OutputNormBlock)
 
 
+class SandwichBlock(Block):
+    """A block with a norm before and after each sublayer: x += post1(mixer(pre1(x))), then
+    x += post2(feed_forward(pre2(x))). The norms before are `Norm`s of the residual, those after
+    parts with `add(ctx, residual, y)` (they norm y and add it into the 32-bit residual; a
+    sparse feed-forward's weighted rows are summed by the same kernel). `feed_forward` may be
+    None (a layer with a mixer only)."""
+
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, mixer_out_norm: Part,
+                 ff_norm: Optional[Norm] = None, feed_forward: Optional[FeedForward] = None,
+                 ff_out_norm: Optional[Part] = None):
+        if (feed_forward is None) != (ff_norm is None) or (feed_forward is None) != (ff_out_norm is None):
+            raise ValueError("a feed-forward and its two norms come together or not at all")
+        self.mixer_norm, self.mixer, self.mixer_out_norm = mixer_norm, mixer, mixer_out_norm
+        self.ff_norm, self.feed_forward, self.ff_out_norm = ff_norm, feed_forward, ff_out_norm
+
+    def children(self) -> List[Part]:
+        return [p for p in (self.mixer_norm, self.mixer, self.mixer_out_norm, self.ff_norm,
+                            self.feed_forward, self.ff_out_norm) if p is not None]
+
+    def forward(self, ctx: StepContext, residual, pending, call: CallInfo):
+        h = self.mixer_norm.forward(ctx, residual, pending)
+        self.mixer_out_norm.add(ctx, residual, self.mixer.forward(ctx, h, residual, call))
+        if self.feed_forward is not None:
+            h = self.ff_norm.forward(ctx, residual, None)
+            y = self.feed_forward.forward(ctx, h, residual)
+            if y is None:
+                raise ValueError("a feed-forward between two norms hands its rows back")
+            self.ff_out_norm.add(ctx, residual, y)
+        return None
+
+
+register_part("block", "sandwich", SandwichBlock)
+
+
 class ParallelBlock(Block):
     """A block whose sublayers run side by side on the same residual: h = norm(x), then
     x += mult (c1 mixer(h) + c2 feed_forward(h2)), where h2 = h, or ff_norm(x) when the block

@@ -12,8 +12,10 @@ latent's space, q'_h = W_uk,h^T q_unrot (a product per head), the attention kern
 q' and the rotated part against the cached rows and sums the latents, and the head's value
 is W_uv,h applied to that sum (another product per head). The gate, one number per head and
 row, scales the head's output in the attention kernel. `position` turns the first
-`position.rot_dim` of the rot_dim rotated numbers (half-split pairs) with its table and
-magnitude. Norm, angles, scores and softmax are 32-bit; q' is kept in 32-bit.
+`position.rot_dim` of the rot_dim rotated numbers (half-split pairs or neighbours, as its
+`pairing` says) with its table and magnitude. Norm, angles, scores and softmax are 32-bit;
+q' is kept in 32-bit. With `q_rank` the queries pass a latent of their own first:
+c_q = rmsnorm(W_dq h) * weight (q_rank numbers, normed in 32-bit), q = W_uq c_q.
 """
 from __future__ import annotations
 
@@ -31,11 +33,17 @@ class LatentAttention(Mixer):
                  kv_rank: int, scale: float, eps: float, position: PositionEncoding,
                  output_gate: bool = True, window: Optional[int] = None,
                  page_size: Optional[int] = None,
-                 names=("q", "dkv", "dkv.norm", "uk", "uv", "g", "o")):
+                 names=("q", "dkv", "dkv.norm", "uk", "uv", "g", "o"),
+                 q_rank: Optional[int] = None, q_names=("dq", "dq.norm", "uq")):
+        """`q_rank`: size of the queries' latent (None: none, `names[0]` projects the queries
+        from the layer's input); `q_names`: what follows the prefix in the names of the down
+        projection, its norm's weight and the up projection of the queries' latent."""
         if position.rot_dim > rot_dim:
             raise ValueError(f"the rotation turns {position.rot_dim} numbers of {rot_dim}")
-        if position.rot_dim and position.pairing != "half":
-            raise ValueError("latent attention turns half-split pairs")
+        self.q_rank = q_rank
+        self.q_names = tuple(q_names)
+        self.w_dq: Optional[torch.Tensor] = None
+        self.q_norm_w: Optional[torch.Tensor] = None
         if not scale > 0:
             raise ValueError(f"scale must be > 0, got {scale}")
         self.prefix = prefix
@@ -68,8 +76,8 @@ class LatentAttention(Mixer):
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         p, n = self.prefix, self.names
+        qn = self.q_names
         specs = {
-            p + n[0]: TensorSpec((self.heads * (self.dim + self.rot_dim), self.hidden)),
             p + n[1]: TensorSpec((self.kv_rank + self.rot_dim, self.hidden)),
             p + n[2]: TensorSpec((self.kv_rank,), "gain"),
             p + n[3]: TensorSpec((self.heads * self.dim, self.kv_rank)),
@@ -78,12 +86,24 @@ class LatentAttention(Mixer):
         }
         if self.output_gate:
             specs[p + n[5]] = TensorSpec((self.heads, self.hidden))
+        q_width = self.heads * (self.dim + self.rot_dim)
+        if self.q_rank is None:
+            specs[p + n[0]] = TensorSpec((q_width, self.hidden))
+        else:
+            specs[p + qn[0]] = TensorSpec((self.q_rank, self.hidden))
+            specs[p + qn[1]] = TensorSpec((self.q_rank,), "gain")
+            specs[p + qn[2]] = TensorSpec((q_width, self.q_rank))
         return specs
 
     def bind(self, w: WeightBinder) -> None:
         p, n = self.prefix, self.names
         lat = self.kv_rank + self.rot_dim
-        self.w_q = w.matrix(p + n[0])
+        if self.q_rank is None:
+            self.w_q = w.matrix(p + n[0])
+        else:
+            self.w_dq = w.matrix(p + self.q_names[0])
+            self.q_norm_w = w.float32(p + self.q_names[1])
+            self.w_q = w.matrix(p + self.q_names[2])
         self.w_dkv_g = torch.empty((lat + (self.heads if self.output_gate else 0), self.hidden),
                                    dtype=w.act_dtype, device=w.device)
         w.matrix_into(p + n[1], self.w_dkv_g[:lat])
@@ -101,14 +121,22 @@ class LatentAttention(Mixer):
         cache = call.cache
         T, H, R, rd = ctx.T, self.heads, self.kv_rank, self.rot_dim
         q = ctx.empty((T, H * (self.dim + rd)))
-        ops.linear(x, self.w_q, q)
+        if self.q_rank is None:
+            ops.linear(x, self.w_q, q)
+        else:   # the queries' latent: projected into 32-bit, normed there, then up
+            cq32 = ctx.empty((T, self.q_rank), torch.float32)
+            ops.linear(x, self.w_dq, cq32)
+            cq = ctx.empty((T, self.q_rank))
+            ops.rmsnorm(cq32, self.q_norm_w, self.eps, cq)
+            ops.linear(cq, self.w_q, q)
         dkv_g = ctx.empty((T, self.w_dkv_g.shape[0]))
         ops.linear(x, self.w_dkv_g, dkv_g)
         q_abs = ctx.empty((T, H, R + rd), torch.float32)
         ops.latent_kv_write(dkv_g, q, q_abs, cache["latent"], cache.block_table, ctx, H, self.dim,
                             R, rd, self.norm_w, self.eps, self.position.table(),
                             self.position.rot_dim, getattr(self.position, "magnitude", 1.0),
-                            cache.page_size, write_kv=call.writes_cache)
+                            cache.page_size, write_kv=call.writes_cache,
+                            interleaved=self.position.pairing == "interleaved")
         ops.per_head_linear(q.view(T, H, self.dim + rd), self.w_absorb, q_abs, ctx, self.dim, R)
         mixed = ctx.empty((T, H * R))
         ops.latent_attention(q_abs, cache["latent"], cache.block_table, ctx, H, R, rd,

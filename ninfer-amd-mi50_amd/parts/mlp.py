@@ -19,14 +19,17 @@ from .base import FeedForward, StepContext, WeightBinder
 
 class SwiGLU(FeedForward):
     def __init__(self, prefix: str, hidden: int, inner: int, act: str = "silu", bias: bool = False,
-                 names=("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
+                 names=("gate_proj.weight", "up_proj.weight", "down_proj.weight"),
+                 act_limit: float = 0.0, act_alpha: float = 1.0):
         """`names`: what follows the prefix in the names of the gate's, the other half's and the
-        down product's weights."""
+        down product's weights. `act` 'clamped_swish': g sigmoid(act_alpha g) (u + 1) with g cut
+        at act_limit from above and u to [-act_limit, act_limit]."""
+        self.act_limit, self.act_alpha = float(act_limit), float(act_alpha)
         self.prefix = prefix
         self.names = tuple(names)
         self.hidden = hidden
         self.inner = inner
-        self.act = act   # the gate's activation, by config.json's name: 'silu' | 'gelu_pytorch_tanh'
+        self.act = act   # the gate's activation: 'silu' | 'gelu_pytorch_tanh' | 'clamped_swish'
         self.bias = bias   # gate_proj.bias, up_proj.bias [inner] and down_proj.bias [hidden] are read
         self.w_gate_up: Optional[torch.Tensor] = None
         self.w_down: Optional[torch.Tensor] = None
@@ -63,7 +66,11 @@ class SwiGLU(FeedForward):
 
     def gate_up(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
         h = ctx.empty((x.shape[0], self.inner))
-        ctx.ops.swiglu_linear(x, self.w_gate_up, h, act=self.act, bias=self.b_gate_up)
+        if self.act == "clamped_swish":
+            ctx.ops.swiglu_linear(x, self.w_gate_up, h, act=self.act, bias=self.b_gate_up,
+                                  limit=self.act_limit, alpha=self.act_alpha)
+        else:
+            ctx.ops.swiglu_linear(x, self.w_gate_up, h, act=self.act, bias=self.b_gate_up)
         return h
 
     def down(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:

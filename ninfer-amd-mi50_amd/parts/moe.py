@@ -35,13 +35,17 @@ class TopKRouter(Part):
                  score: str = "softmax", scale: float = 1.0, choice_bias: bool = False,
                  n_group: int = 0, topk_group: int = 0, group_top: int = 1,
                  renorm_eps: float = 0.0, leaf: str = "weight", weightless: int = 0,
-                 choice_bias_leaf: str = "choice_bias"):
+                 choice_bias_leaf: str = "choice_bias", logit_bias_leaf: Optional[str] = None):
         """`group_top`: a group's score in the group-limited choice is the sum of its group_top
         largest scores (1: its largest). `renorm_eps` is added to the sum of the chosen scores
         before the division. `leaf`: what follows the prefix in the weight's name,
         `choice_bias_leaf` in the bias's. `weightless`: the last so many of the `experts`
         router outputs stand for experts without weights (they are scored, grouped and chosen
-        like the others; the grouped products pass their rows over)."""
+        like the others; the grouped products pass their rows over). `logit_bias_leaf`: the
+        name (after the prefix) of a bias [experts] that is added to the logits themselves, so
+        that it enters the scores and the weights as well as the choice."""
+        self.logit_bias_leaf = logit_bias_leaf
+        self.logit_bias: Optional[torch.Tensor] = None
         if top_k > experts:
             raise ValueError(f"top_k ({top_k}) exceeds the number of experts ({experts})")
         if score not in ("softmax", "sigmoid"):
@@ -74,16 +78,20 @@ class TopKRouter(Part):
         specs = {self.prefix + self.leaf: TensorSpec((self.experts, self.hidden))}
         if self.has_choice_bias:
             specs[self.prefix + self.choice_bias_leaf] = TensorSpec((self.experts,), role="bias")
+        if self.logit_bias_leaf:
+            specs[self.prefix + self.logit_bias_leaf] = TensorSpec((self.experts,), role="bias")
         return specs
 
     def bind(self, w: WeightBinder) -> None:
         self.weight = w.matrix(self.prefix + self.leaf)
         if self.has_choice_bias:
             self.choice_bias = w.float32(self.prefix + self.choice_bias_leaf)
+        if self.logit_bias_leaf:
+            self.logit_bias = w.float32(self.prefix + self.logit_bias_leaf)
 
     def logits(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
         out = ctx.empty((x.shape[0], self.experts), torch.float32)
-        ctx.ops.linear(x, self.weight, out)
+        ctx.ops.linear(x, self.weight, out, bias=self.logit_bias)
         return out
 
     def route(self, ctx: StepContext, logits: torch.Tensor) -> "Routing":
@@ -194,7 +202,7 @@ class SparseMoE(FeedForward):
                  renorm: bool, shared_inner: int = 0, act: str = "silu", router=None, names=None,
                  identity: int = 0, act_limit: float = 0.0, act_alpha: float = 1.0):
         """`router`: further parameters of `TopKRouter` (score, scale, n_group, topk_group,
-        group_top, renorm_eps, choice_bias, choice_bias_leaf). `identity`: the router has so
+        group_top, renorm_eps, choice_bias, choice_bias_leaf, logit_bias_leaf). `identity`: the router has so
         many outputs beyond the `experts` with weights; the expert of such an output hands its
         input back (times the weight). `act_limit`, `act_alpha`: see `RoutedExperts`."""
         self.prefix = prefix

@@ -13,6 +13,11 @@ NTK-by-parts rule known as YaRN): with d(t) = rot_dim ln(original / (2 pi t)) /
 and r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair i turns at
 f_i / factor * r_i + f_i * (1 - r_i), and cosine and sine are both multiplied by
 `magnitude` = 0.1 ln(factor) + 1.
+
+A `scaling` with the keys {factor, original, low, high} slows pairs down by their wavelength
+l_i = 2 pi / f_i instead: f_i stays where l_i < original / high, becomes f_i / factor where
+l_i > original / low, and between the two, with s = (original / l_i - low) / (high - low),
+(1 - s) f_i / factor + s f_i; cosine and sine keep their size.
 """
 from __future__ import annotations
 
@@ -30,7 +35,9 @@ class Rotary(PositionEncoding):
                  scaling: Optional[Dict[str, float]] = None):
         """`scaling`: None, or {'factor', 'original', 'fast', 'slow'}: the stretch, the trained
         context, and the turns over that context above which a pair is left alone (`fast`)
-        and below which it is stretched in full (`slow`)."""
+        and below which it is stretched in full (`slow`); or {'factor', 'original', 'low',
+        'high'}: the same bounds given as wavelengths, original / high and original / low, with
+        the blend linear in the turns and cosine and sine left as they are."""
         if rot_dim % 2:
             raise ValueError(f"rotary dimension must be even, got {rot_dim}")
         if pairing not in ("half", "interleaved"):
@@ -40,7 +47,15 @@ class Rotary(PositionEncoding):
         self.theta = float(theta)
         self.scaling = None
         self.magnitude = 1.0   # factor on cosine and sine
-        if scaling is not None:
+        self.bands = None
+        if scaling is not None and "low" in scaling and "high" in scaling:
+            missing = [k for k in ("factor", "original") if k not in scaling]
+            if missing:
+                raise ValueError(f"rotary scaling lacks {missing}")
+            self.bands = {k: float(scaling[k]) for k in ("factor", "original", "low", "high")}
+            if not self.bands["factor"] > 0 or not self.bands["high"] > self.bands["low"] > 0:
+                raise ValueError("rotary scaling needs factor > 0 and high > low > 0")
+        elif scaling is not None:
             missing = [k for k in ("factor", "original", "fast", "slow") if k not in scaling]
             if missing:
                 raise ValueError(f"rotary scaling lacks {missing}")
@@ -63,6 +78,17 @@ class Rotary(PositionEncoding):
             for i in range(n // 2):
                 ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
                 vals[i] = vals[i] / sc["factor"] * ramp + vals[i] * (1.0 - ramp)
+        if self.bands is not None:
+            b = self.bands
+            for i, f in enumerate(vals):
+                wave = 2.0 * math.pi / f
+                if wave < b["original"] / b["high"]:
+                    continue
+                if wave > b["original"] / b["low"]:
+                    vals[i] = f / b["factor"]
+                else:
+                    s = (b["original"] / wave - b["low"]) / (b["high"] - b["low"])
+                    vals[i] = (1.0 - s) * f / b["factor"] + s * f
         return torch.tensor(vals, dtype=torch.float64).to(torch.float32)
 
     def bind(self, w: WeightBinder) -> None:
