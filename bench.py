@@ -35,6 +35,13 @@ the same for Fopinex (gated parallel blocks of attention without a softmax or ga
 attention and routed experts beside identity experts) beside a Qwen2-MoE model of the same
 width, depth, heads and experts.
 
+    python bench.py --scenario designs --design tuzapel [--sizes small,medium] [--only tuzapel|sparse]
+
+the same for Tuzapel (layer norms before and after every sublayer; latent attention with a
+query latent, or windowed attention with a convolution on q, k and v, normed heads, a sink
+and layers that read another layer's keys and values; a clamped gated feed-forward, dense or
+as routed experts) beside a Qwen2-MoE model of the same width, depth, heads, window and experts.
+
     python bench.py --scenario long [--model 57b-a14b] [--requests 8] [--prompt 32768] [--new 256]
 
 is another measurement with a JSON line of its own: the scheduler serves
@@ -97,7 +104,7 @@ def main() -> int:
     ap.add_argument("--scenario", default="decode", choices=["decode", "long", "designs"])
     ap.add_argument("--sizes", default="small,medium",
                     help="--scenario designs: which of the layer sizes to run (small, medium)")
-    ap.add_argument("--design", default="getodra", choices=["getodra", "sosepel", "fopinex"],
+    ap.add_argument("--design", default="getodra", choices=["getodra", "sosepel", "fopinex", "tuzapel"],
                     help="--scenario designs: the design to run beside the closest model the engine had")
     ap.add_argument("--only", default="", help="--scenario designs: run this one of the two models only")
     ap.add_argument("--requests", type=int, default=8, help="--scenario long: concurrent requests")
@@ -609,24 +616,80 @@ def sparse_for_fopinex_config(z: dict) -> dict:
                 vocab_size=z["vocab"], hidden_act="silu", use_sliding_window=False)
 
 
+TUZAPEL_SIZES = {
+    # width, layers (of every four: latent attention, windowed attention, windowed attention on
+    # the layer before's keys and values, windowed attention; feed-forwards in turn routed and
+    # dense), query and kv heads, sizes of a key and a value, window, taps, the latent
+    # attention's sizes, experts
+    "small": dict(width=1024, layers=8, heads=8, kv_heads=2, dim=128, vdim=128, window=1024, taps=4,
+                  lat_dim=96, lat_rot=32, lat_vdim=64, rank=256, q_rank=384, ff=2816, experts=16,
+                  top=2, expert_ff=704, vocab=32000, positions=4096),
+    "medium": dict(width=2048, layers=8, heads=16, kv_heads=4, dim=128, vdim=128, window=1024, taps=4,
+                   lat_dim=64, lat_rot=64, lat_vdim=128, rank=512, q_rank=768, ff=5632, experts=32,
+                   top=4, expert_ff=1408, vocab=32000, positions=4096),
+}
+
+
+def tuzapel_config(z: dict) -> dict:
+    rot = {"base": 500000.0, "dims": z["dim"] // 2,
+           "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 2048}}
+    attention = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["vdim"],
+                 "scale": z["dim"] ** -0.5, "conv": z["taps"], "mask": {"size": z["window"]}, "rot": rot}
+    latent = {"heads": z["heads"], "dim": z["lat_dim"], "rot_dim": z["lat_rot"], "vdim": z["lat_vdim"],
+              "kv_rank": z["rank"], "q_rank": z["q_rank"], "scale": (z["lat_dim"] + z["lat_rot"]) ** -0.5,
+              "rot": {"base": 10000.0, "dims": z["lat_rot"]}}
+    moe = {"kind": "moe", "expert": {"ff": z["expert_ff"], "limit": 7.0},
+           "router": {"experts": z["experts"], "top": z["top"]}}
+    dense = {"kind": "dense", "ff": z["ff"], "limit": 7.0}
+    layers = []
+    for i in range(z["layers"]):
+        mlp = moe if i % 2 else dense
+        if i % 4 == 0:
+            layers.append({"type": "latent_attention", "mixer": latent, "mlp": mlp})
+        elif i % 4 == 2:
+            layers.append({"type": "attention", "mixer": dict(attention, kv_from=i - 1), "mlp": mlp})
+        else:
+            layers.append({"type": "attention", "mixer": attention, "mlp": mlp})
+    return {"architecture": "Tuzapel", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6},
+            "logit_softcap": 30.0, "layers": layers}
+
+
+def sparse_for_tuzapel_config(z: dict) -> dict:
+    """The closest model the engine had: Qwen2-MoE blocks (rotary attention with as many query
+    and kv heads of the same size behind the same window, routed experts of the same size on the
+    same layers and a dense feed-forward on the others, no shared expert) of the same width and
+    depth."""
+    return dict(CONFIG_C, num_hidden_layers=z["layers"], hidden_size=z["width"],
+                num_attention_heads=z["heads"], num_key_value_heads=z["kv_heads"], head_dim=z["dim"],
+                intermediate_size=z["ff"], num_experts=z["experts"], num_experts_per_tok=z["top"],
+                moe_intermediate_size=z["expert_ff"], shared_expert_intermediate_size=0,
+                mlp_only_layers=[i for i in range(z["layers"]) if i % 2 == 0], decoder_sparse_step=1,
+                vocab_size=z["vocab"], hidden_act="silu", use_sliding_window=True,
+                sliding_window=z["window"], max_window_layers=0)
+
+
 def designs_scenario(args) -> int:
     import torch
     from ninfer_amd import Chunk, EngineOptions, random_model
     sosepel = args.design == "sosepel"
+    tuzapel = args.design == "tuzapel"
 
     gen = torch.Generator().manual_seed(11)
     fopinex = args.design == "fopinex"
     out = {"metric": "prefill and decode throughput, " + ("Sosepel beside a Qwen2-MoE model" if sosepel
                      else "Fopinex beside a Qwen2-MoE model" if fopinex
+                     else "Tuzapel beside a Qwen2-MoE model" if tuzapel
                      else "Getodra beside a dense model") + " of equal size",
            "unit": "tok/s", "n_gpus": 1, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
            "data": "synthetic", "sizes": {}}
     for size in args.sizes.split(","):
-        z = (SOSEPEL_SIZES if sosepel else FOPINEX_SIZES if fopinex else DESIGN_SIZES)[size]
+        z = (SOSEPEL_SIZES if sosepel else FOPINEX_SIZES if fopinex else TUZAPEL_SIZES if tuzapel
+             else DESIGN_SIZES)[size]
         ctx = z["positions"]
         row = {"shape": z}
         pairs = (("sosepel", sosepel_config(z)), ("sparse", sparse_config(z))) if sosepel else \
             (("fopinex", fopinex_config(z)), ("sparse", sparse_for_fopinex_config(z))) if fopinex else \
+            (("tuzapel", tuzapel_config(z)), ("sparse", sparse_for_tuzapel_config(z))) if tuzapel else \
             (("getodra", getodra_config(z)), ("dense", dense_config(z)))
         for name, raw in pairs:
             if args.only and name != args.only:

@@ -47,7 +47,7 @@ class PlainOps:
             x = x + _f(pos_table[positions.long()])
         out.copy_(x)
 
-    def rmsnorm(self, x, gain, eps, out, delta=None, rows=None, rows_sum=None):
+    def rmsnorm(self, x, gain, eps, out, delta=None, rows=None, rows_sum=None, center=False):
         extra = None
         if delta is not None:
             extra = _f(delta)
@@ -63,8 +63,118 @@ class PlainOps:
             v = x[rows.long()]
             if extra is not None:
                 v = v + extra[rows.long()]
+        if center:
+            v = v - v.mean(-1, keepdim=True)
         ms = (v * v).sum(-1, keepdim=True) / v.shape[-1]
         out.copy_((v * torch.rsqrt(ms + eps) * gain).to(out.dtype))
+
+    def norm_add(self, residual, y, gain, eps, center=False, weights=None):
+        v = _f(y)
+        if weights is not None:
+            t, k = weights.shape
+            v = (v.view(t, k, -1) * weights[:, :, None]).sum(1)
+        if center:
+            v = v - v.mean(-1, keepdim=True)
+        residual += v * torch.rsqrt((v * v).mean(-1, keepdim=True) + eps) * gain
+
+    @staticmethod
+    def _turn(x, positions, inv_freq, rot_dim, interleaved):
+        """x [T, heads, d]: the first rot_dim numbers of every head turned by pos * inv_freq."""
+        if not rot_dim:
+            return x
+        phi = positions.to(torch.float32)[:, None] * inv_freq[None, :]
+        c, s = torch.cos(phi)[:, None, :], torch.sin(phi)[:, None, :]
+        x = x.clone()
+        if interleaved:
+            a, b = x[..., 0:rot_dim:2].clone(), x[..., 1:rot_dim:2].clone()
+            x[..., 0:rot_dim:2] = a * c - b * s
+            x[..., 1:rot_dim:2] = b * c + a * s
+        else:
+            half = rot_dim // 2
+            a, b = x[..., :half].clone(), x[..., half:rot_dim].clone()
+            x[..., :half] = a * c - b * s
+            x[..., half:rot_dim] = b * c + a * s
+        return x
+
+    def qkv_conv(self, u, w_conv, state, ctx, q_out, heads, kv_heads, dim, vdim, k_pool, v_pool,
+                 block_table, page_size, q_norm=None, k_norm=None, norm_eps=0.0, inv_freq=None,
+                 rot_dim=0, interleaved=False):
+        t, ch = u.shape
+        y = _f(u).clone()
+        if w_conv is not None:
+            taps = w_conv.shape[1]
+            start, slots = ctx.seq_row_start.tolist(), ctx.seq_slots.tolist()
+            for s in range(ctx.S):
+                rows = _f(u[start[s]:start[s + 1]])
+                if taps > 1:
+                    held = state[slots[s], :(taps - 1) * ch].view(taps - 1, ch)
+                    ext = torch.cat([held, rows], 0)
+                    state[slots[s], :(taps - 1) * ch] = ext[ext.shape[0] - (taps - 1):].reshape(-1)
+                else:
+                    ext = rows
+                n = rows.shape[0]
+                acc = torch.zeros_like(rows)
+                for j in range(taps):
+                    acc += w_conv[:, j][None, :] * ext[j:j + n]
+                y[start[s]:start[s + 1]] = acc
+        nq, nk = heads * dim, kv_heads * dim
+
+        def normed(x, gain):
+            if gain is None:
+                return x
+            return x * torch.rsqrt((x * x).mean(-1, keepdim=True) + norm_eps) * gain
+        q = self._turn(normed(y[:, :nq].view(t, heads, dim), q_norm), ctx.positions, inv_freq,
+                       rot_dim, interleaved)
+        q_out.copy_(q.reshape(t, nq).to(q_out.dtype))
+        if not kv_heads:
+            return
+        k = self._turn(normed(y[:, nq:nq + nk].view(t, kv_heads, dim), k_norm), ctx.positions,
+                       inv_freq, rot_dim, interleaved)
+        v = y[:, nq + nk:].view(t, kv_heads, vdim)
+        pos = ctx.positions.long()
+        page = block_table[ctx.row_seq.long(), pos // page_size].long()
+        assert (page >= 0).all(), "write into a page that is not held"
+        k_pool[page, :, pos % page_size, :] = k.to(k_pool.dtype)
+        v_pool[page, :, pos % page_size, :] = v.to(v_pool.dtype)
+
+    def latent_kv_write(self, dkv, q, q_abs, pool, block_table, ctx, heads, dim, rank, rot_dim,
+                        norm_w, eps, freq, rot_n, magnitude, page_size, write_kv=True,
+                        interleaved=False):
+        assert magnitude == 1.0, "the stand-in turns without a magnitude"
+        t = ctx.T
+        c = _f(dkv[:, :rank])
+        c = c * torch.rsqrt((c * c).mean(-1, keepdim=True) + eps) * norm_w
+        kr = self._turn(_f(dkv[:, rank:rank + rot_dim]).view(t, 1, rot_dim), ctx.positions, freq,
+                        rot_n, interleaved)[:, 0]
+        if write_kv:
+            pos = ctx.positions.long()
+            page = block_table[ctx.row_seq.long(), pos // page_size].long()
+            assert (page >= 0).all(), "write into a page that is not held"
+            pool[page, pos % page_size, :] = torch.cat([c, kr], -1).to(pool.dtype)
+        qr = self._turn(_f(q).view(t, heads, dim + rot_dim)[:, :, dim:], ctx.positions, freq, rot_n,
+                        interleaved)
+        q_abs[:, :, rank:] = qr
+
+    def head_index(self, ctx, heads):
+        return None, None
+
+    def per_head_linear(self, x, w, out, ctx, k, n):
+        out[:, :, :n] = torch.einsum("thk,hnk->thn", _f(x[:, :, :k]), _f(w)).to(out.dtype)
+
+    def latent_attention(self, q_abs, pool, block_table, ctx, heads, rank, rot_dim, page_size,
+                         scale, out, gate=None, window=None):
+        pos, seq = ctx.positions.tolist(), ctx.row_seq.tolist()
+        for r in range(ctx.T):
+            lo = max(0, pos[r] - window + 1) if window else 0
+            js = torch.arange(lo, pos[r] + 1)
+            pages = block_table[seq[r], js // page_size].long()
+            assert (pages >= 0).all(), "read of a page that is not held"
+            rows = _f(pool[pages, js % page_size, :])          # [n, rank + rot_dim]
+            p = torch.softmax(rows @ q_abs[r].T * scale, 0)     # [n, heads]
+            o = p.T @ rows[:, :rank]
+            if gate is not None:
+                o = o * torch.sigmoid(_f(gate[r]))[:, None]
+            out[r] = o.reshape(-1).to(out.dtype)
 
     def qkv_rope(self, x, w_qkv, bias, qkv, positions, row_seq, inv_freq, rot_dim, n_q, n_kv,
                  head_dim, k_pool, v_pool, block_table, page_size, write_kv=True,
@@ -225,8 +335,9 @@ class PlainOps:
         self.moe_align(r.ids, experts, r.offsets, r.order, tiles=r, weightless=weightless)
 
     def paged_attention(self, qkv, k_pool, v_pool, block_table, ctx, n_q, n_kv, head_dim,
-                        page_size, window, scale, out, slopes=None):
+                        page_size, window, scale, out, slopes=None, vdim=None, sink=False):
         t = qkv.shape[0]
+        vdim = head_dim if vdim is None else vdim
         q = _f(qkv[:, :n_q * head_dim]).view(t, n_q, head_dim)
         group = n_q // n_kv
         pos = ctx.positions.tolist()
@@ -243,9 +354,10 @@ class PlainOps:
                 s = (k[:, g, :] @ q[r, h]) * scale
                 if slopes is not None:
                     s = s + float(slopes[h]) * (js - pos[r]).float().to(s.device)
-                p = torch.exp(s - s.max())
-                p = p / p.sum()
-                out[r, h * head_dim:(h + 1) * head_dim] = (p @ v[:, g, :]).to(out.dtype)
+                top = torch.clamp(s.max(), min=0.0) if sink else s.max()
+                p = torch.exp(s - top)
+                p = p / (p.sum() + (torch.exp(-top) if sink else 0.0))
+                out[r, h * vdim:(h + 1) * vdim] = (p @ v[:, g, :]).to(out.dtype)
 
     # ---- parallel sublayers, hashed pairs, differential attention ------------------------------
     def embed_pairs(self, ctx, table, out, scale=1.0, pair_table=None, buckets=0, mul_prev=0,

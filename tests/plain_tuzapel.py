@@ -53,7 +53,7 @@ def frequencies(rot: dict) -> torch.Tensor:
 def rotate(x: torch.Tensor, pos: torch.Tensor, rot: dict, pairing: str) -> torch.Tensor:
     """x [n, heads, d]: the first rot.dims numbers of every head turn by pos * f_i; pair i is
     (2i, 2i + 1) when `pairing` is 'interleaved', (i, i + dims / 2) when 'half'."""
-    dims = rot["dims"]
+    dims = (rot or {}).get("dims", 0)
     if not dims:
         return x
     ang = pos.to(D)[:, None] * frequencies(rot)[None, :]          # [n, dims / 2]
@@ -112,12 +112,15 @@ def latent_attention(w, prefix: str, mixer: dict, h: torch.Tensor, eps: float) -
     n = h.shape[0]
     H, d, rd, dv, R = mixer["heads"], mixer["dim"], mixer["rot_dim"], mixer["vdim"], mixer["kv_rank"]
     pos = torch.arange(n)
-    cq = rms_norm(lin(w, prefix + "dq", h), w[prefix + "dq.norm"], eps)
-    q = lin(w, prefix + "uq", cq).reshape(n, H, d + rd)
-    q_plain, q_rot = q[..., :d], rotate(q[..., d:], pos, mixer["rot"], "interleaved")
+    if mixer.get("q_rank"):
+        cq = rms_norm(lin(w, prefix + "dq", h), w[prefix + "dq.norm"], eps)
+        q = lin(w, prefix + "uq", cq).reshape(n, H, d + rd)
+    else:
+        q = lin(w, prefix + "q", h).reshape(n, H, d + rd)
+    q_plain, q_rot = q[..., :d], rotate(q[..., d:], pos, mixer.get("rot"), "interleaved")
     ckv = lin(w, prefix + "dkv", h)
     c = rms_norm(ckv[:, :R], w[prefix + "dkv.norm"], eps)
-    k_rot = rotate(ckv[:, None, R:], pos, mixer["rot"], "interleaved")[:, 0]      # [n, rd]
+    k_rot = rotate(ckv[:, None, R:], pos, mixer.get("rot"), "interleaved")[:, 0]      # [n, rd]
     k_plain = lin(w, prefix + "uk", c).reshape(n, H, d)
     v = lin(w, prefix + "uv", c).reshape(n, H, dv)
     vis = visible(n, None)
@@ -132,18 +135,23 @@ def window_keys_values(w, prefix: str, mixer: dict, h: torch.Tensor, eps: float)
     """k [n, G, dim] after convolution, norm and rotation; v [n, G, vdim] after convolution."""
     n = h.shape[0]
     G, d, dv = mixer["kv_heads"], mixer["dim"], mixer["vdim"]
-    k = short_conv(lin(w, prefix + "k", h), w[prefix + "k.conv"]).reshape(n, G, d)
-    v = short_conv(lin(w, prefix + "v", h), w[prefix + "v.conv"]).reshape(n, G, dv)
+    k, v = lin(w, prefix + "k", h), lin(w, prefix + "v", h)
+    if mixer.get("conv"):
+        k, v = short_conv(k, w[prefix + "k.conv"]), short_conv(v, w[prefix + "v.conv"])
+    k, v = k.reshape(n, G, d), v.reshape(n, G, dv)
     k = rms_norm(k, w[prefix + "k.norm"], eps)
-    k = rotate(k, torch.arange(n), mixer["rot"], "half")
+    k = rotate(k, torch.arange(n), mixer.get("rot"), "half")
     return k, v
 
 
 def window_attention(w, prefix: str, mixer: dict, h: torch.Tensor, eps: float, kv) -> torch.Tensor:
     n = h.shape[0]
     H, G, d, dv = mixer["heads"], mixer["kv_heads"], mixer["dim"], mixer["vdim"]
-    q = short_conv(lin(w, prefix + "q", h), w[prefix + "q.conv"]).reshape(n, H, d)
-    q = rotate(rms_norm(q, w[prefix + "q.norm"], eps), torch.arange(n), mixer["rot"], "half")
+    q = lin(w, prefix + "q", h)
+    if mixer.get("conv"):
+        q = short_conv(q, w[prefix + "q.conv"])
+    q = q.reshape(n, H, d)
+    q = rotate(rms_norm(q, w[prefix + "q.norm"], eps), torch.arange(n), mixer.get("rot"), "half")
     k, v = kv
     vis = visible(n, (mixer.get("mask") or {}).get("size"))
     per = H // G
