@@ -22,7 +22,9 @@
 // Single rows (decode steps): a block of two waves owns one row and one kv head, the query heads
 // of the kv head (at most 32) are the tile's rows, so that the keys and values of the kv head
 // are read once for all of them; wave w takes keys 32 w .. + 31 of every tile with a running
-// maximum, sum and output of its own, and the two meet through LDS at the end.
+// maximum, sum and output of its own, and the two meet through LDS at the end. When rows and
+// kv heads alone do not fill the GPU, a row's visible keys are cut into chunks of whole tiles
+// over several blocks, whose records a second kernel merges.
 //
 // No load stands under a condition: a key that is not there (beyond the last row's position,
 // or before the first key any row of the tile sees, whose page a window may have given back)
@@ -283,8 +285,13 @@ __global__ __launch_bounds__(256, 2) void attention_tiles_kernel(AttnArgs a, int
     }
 }
 
+// `tiles_per_chunk`, `n_chunks`: the visible keys of a row are cut into chunks of so many tiles
+// (counted from the tile that holds the row's first visible key), one block each
+// (blockIdx.z), when rows and kv heads alone do not fill the GPU; every block then leaves a
+// record {m, l, o[Dv]} per head (m in units of log 2) that the merge kernel puts together.
 template <int KS, int DB>
-__global__ __launch_bounds__(128, 4) void attention_tiles_heads_kernel(AttnArgs a) {
+__global__ __launch_bounds__(128, 2) void attention_tiles_heads_kernel(AttnArgs a, int tiles_per_chunk,
+                                                                    int n_chunks) {
   using Mover = TileMover<KS, DB, 128>;
   constexpr int KROW = Mover::KROW, VROW = Mover::VROW, TILE = Mover::TILE;
   extern __shared__ __attribute__((aligned(16))) unsigned short lds[];
@@ -292,12 +299,22 @@ __global__ __launch_bounds__(128, 4) void attention_tiles_heads_kernel(AttnArgs 
   const int tid = threadIdx.x, lane = tid & 63, kb = tid >> 6;
   const int c = lane & 31, hi = lane >> 5;
   const int hpg = a.Hq / a.Hkv;
-  const int t = blockIdx.x, g = blockIdx.y;
+  const int t = blockIdx.x, g = blockIdx.y, ch = blockIdx.z;
   const int pos = a.positions[t];
   const int first = a.window > 0 ? max(0, pos - a.window + 1) : 0;
   const int dim = a.D, vdim = a.Dv;
   const bool q_valid = c < hpg;
   const int h = g * hpg + (q_valid ? c : 0);
+  const int kt0 = first / 64 + ch * tiles_per_chunk;
+  const int n_kt = min(pos / 64 + 1, kt0 + tiles_per_chunk);
+  float* rec = n_chunks > 1 ? a.workspace + (((int64_t)t * a.Hq + h) * n_chunks + ch) * (2 + vdim) : nullptr;
+  if (kt0 >= n_kt) {   // nothing of this chunk is visible: records that count for nothing
+    if (q_valid && hi == 0 && kb == 0) {
+      rec[0] = -1e30f;
+      rec[1] = 0.f;
+    }
+    return;
+  }
   const int* bt = a.block_table + (int64_t)a.row_seq[t] * a.bt_stride;
   const int ps_shift = __builtin_ctz(a.page_size), ps_mask = a.page_size - 1;
   const unsigned short* kpool = (const unsigned short*)a.kpool;
@@ -324,12 +341,12 @@ __global__ __launch_bounds__(128, 4) void attention_tiles_heads_kernel(AttnArgs 
   for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int v = 0; v < 16; ++v) o[db][v] = 0.f;
-  // the sink counts once: in the first wave's sum
-  float m = a.sink && kb == 0 ? 0.f : -1e30f, l = a.sink && kb == 0 ? 1.f : 0.f;
+  // the sink counts once: in the first wave's sum of the first chunk
+  const bool with_sink = a.sink && kb == 0 && ch == 0;
+  float m = with_sink ? 0.f : -1e30f, l = with_sink ? 1.f : 0.f;
   const int s16 = lane & 15, q4 = lane >> 4;
   const int v_lane = (4 * hi + s16 / 4) * VROW + 16 * (q4 & 1) + 4 * (s16 & 3);
 
-  const int kt0 = first / 64, n_kt = pos / 64 + 1;
   mv.load(kpool, vpool, bt, ps_shift, ps_mask, a.page_size, a.Hkv, g, dim, vdim, kt0 * 64, first, pos);
   __syncthreads();
   for (int kt = kt0; kt < n_kt; ++kt) {
@@ -362,6 +379,24 @@ __global__ __launch_bounds__(128, 4) void attention_tiles_heads_kernel(AttnArgs 
   const float m2 = x_s[lane], l2 = x_s[64 + lane];
   const float mm = fmaxf(m, m2);
   const float f1 = __builtin_amdgcn_exp2f(m - mm), f2 = __builtin_amdgcn_exp2f(m2 - mm);
+  if (rec) {   // one chunk of several: the record, unnormalised
+    if (hi == 0) {
+      rec[0] = mm;
+      rec[1] = l * f1 + l2 * f2;
+    }
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int v4 = 0; v4 < 4; ++v4) {
+        const int col = 32 * db + 8 * v4 + 4 * hi;
+        if (col < vdim) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            rec[2 + col + e] = o[db][4 * v4 + e] * f1 + x_s[(2 + db * 16 + 4 * v4 + e) * 64 + lane] * f2;
+        }
+      }
+    return;
+  }
   const float r = 1.f / (l * f1 + l2 * f2);
   unsigned short* orow = (unsigned short*)a.out + ((int64_t)t * a.Hq + h) * vdim;
 #pragma unroll
@@ -377,6 +412,54 @@ __global__ __launch_bounds__(128, 4) void attention_tiles_heads_kernel(AttnArgs 
         *(uint2*)(orow + col) = w.u;
       }
     }
+}
+
+// The records of a row and head put together: out = sum_c o_c 2^(m_c - m) / sum_c l_c 2^(m_c - m).
+__global__ __launch_bounds__(64) void attention_tiles_merge_kernel(AttnArgs a, int n_chunks) {
+  const int th = blockIdx.x, lane = threadIdx.x;
+  const int vdim = a.Dv;
+  const float* rec = a.workspace + (int64_t)th * n_chunks * (2 + vdim);
+  float mm = -1e30f;
+  for (int c = 0; c < n_chunks; ++c) mm = fmaxf(mm, rec[c * (2 + vdim)]);
+  float l = 0.f, acc[2] = {0.f, 0.f};
+  for (int c = 0; c < n_chunks; ++c) {
+    const float* r = rec + c * (2 + vdim);
+    if (r[1] == 0.f) continue;   // a chunk with no visible key holds no output
+    const float f = __builtin_amdgcn_exp2f(r[0] - mm);
+    l += r[1] * f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int d = lane + 64 * i;
+      if (d < vdim) acc[i] += r[2 + d] * f;
+    }
+  }
+  const float inv = 1.f / l;
+  __bf16* orow = (__bf16*)a.out + (int64_t)th * vdim;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int d = lane + 64 * i;
+    if (d < vdim) orow[d] = (__bf16)(acc[i] * inv);
+  }
+}
+
+// Chunks of the visible keys (whole tiles) so that the launch has about four blocks a CU, at
+// least two tiles a chunk.
+static void heads_plan(const AttnArgs& a, int* tiles_per_chunk, int* n_chunks) {
+  const int span = a.window > 0 && a.window < a.max_kv_len ? a.window : a.max_kv_len;
+  const int tiles = span / 64 + 2;   // a span of keys that starts anywhere in a tile
+  const int blocks = a.T * a.Hkv;
+  const int want = (4 * device_cu_count() + blocks - 1) / blocks;
+  int per = (tiles + want - 1) / want;
+  if (per < 2) per = 2;
+  int n = (tiles + per - 1) / per;
+  // as many chunks as the workspace holds records for; without one, a block walks a row's
+  // keys alone
+  while (n > 1 && (!a.workspace || a.workspace_floats < (int64_t)a.T * a.Hq * n * (2 + a.Dv))) {
+    per = a.workspace ? per + 1 : tiles;
+    n = (tiles + per - 1) / per;
+  }
+  *tiles_per_chunk = per;
+  *n_chunks = n;
 }
 
 bool attention_tiles_takes(const AttnArgs& a) {
@@ -422,8 +505,14 @@ static int launch_heads(const AttnArgs& a, hipStream_t stream) {
   auto kern = attention_tiles_heads_kernel<KS, DB>;
   static bool raised = false;
   if (int rc = raise_lds(kern, lds, &raised)) return rc;
-  kern<<<dim3(a.T, a.Hkv), 128, lds, stream>>>(a);
+  int per, n;
+  heads_plan(a, &per, &n);
+  kern<<<dim3(a.T, a.Hkv, n), 128, lds, stream>>>(a, per, n);
   NINFER_LAUNCH_CHECK();
+  if (n > 1) {
+    attention_tiles_merge_kernel<<<a.T * a.Hq, 64, 0, stream>>>(a, n);
+    NINFER_LAUNCH_CHECK();
+  }
   return 0;
 }
 

@@ -70,46 +70,91 @@ __global__ void short_conv_state_kernel(const float* __restrict__ x, float* __re
 // x += norm(y) g with norm(y) = y rsqrt(mean(y^2) + eps), or with `center` the layer norm
 // (y - mean) rsqrt(mean((y - mean)^2) + eps). y is a row of `y`, or with `w` the weighted sum of
 // k rows, y_r = sum_j w[r, j] y[r k + j] (a sparse feed-forward's chosen experts), formed in
-// 32-bit in the order of j. A thread keeps its (at most 8) numbers of the row in registers.
+// 32-bit in the order of j. A thread keeps its (at most 8) numbers of the row in registers, in
+// groups of VEC consecutive ones (VEC 4: whole 8- and 16-byte loads and stores).
 constexpr int kNormAddPerThread = 8;
-template <typename T>
+template <int VEC>
+__device__ __forceinline__ void na_load(const float* p, float* f) {
+  if constexpr (VEC == 4) {
+    const float4 v = *(const float4*)p;
+    f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+  } else {
+    f[0] = p[0];
+  }
+}
+template <int VEC>
+__device__ __forceinline__ void na_load(const bf16* p, float* f) {
+  if constexpr (VEC == 4) {
+    const uint2 v = *(const uint2*)p;   // four bf16: the upper halves of four floats
+    f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+    f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+  } else {
+    f[0] = to_f32(p[0]);
+  }
+}
+
+template <typename T, int VEC>
 __global__ void norm_add_kernel(float* __restrict__ x, const T* __restrict__ y,
                                 const float* __restrict__ w, int k,
                                 const float* __restrict__ gain, int gain_n, int H, float eps,
                                 int center) {
+  constexpr int G = kNormAddPerThread / VEC;
   __shared__ float red[16];
   const int64_t r = blockIdx.x;
-  float vals[kNormAddPerThread];
+  float vals[G][VEC];
   float sum = 0.f;
 #pragma unroll
-  for (int c = 0; c < kNormAddPerThread; ++c) {
-    const int i = threadIdx.x + c * blockDim.x;
-    float v = 0.f;
+  for (int c = 0; c < G; ++c) {
+    const int i = VEC * (threadIdx.x + c * blockDim.x);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) vals[c][e] = 0.f;
     if (i < H) {
       if (w) {
-        for (int j = 0; j < k; ++j) v = fmaf(w[r * k + j], to_f32(y[(r * k + j) * H + i]), v);
+        for (int j = 0; j < k; ++j) {
+          float yv[VEC];
+          na_load<VEC>(y + (r * k + j) * H + i, yv);
+          const float wj = w[r * k + j];
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) vals[c][e] = fmaf(wj, yv[e], vals[c][e]);
+        }
       } else {
-        v = to_f32(y[r * H + i]);
+        na_load<VEC>(y + r * H + i, vals[c]);
       }
     }
-    vals[c] = v;
-    sum += v;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) sum += vals[c][e];
   }
   const float mean = center ? block_sum(sum, red) / (float)H : 0.f;
   float ss = 0.f;
 #pragma unroll
-  for (int c = 0; c < kNormAddPerThread; ++c) {
-    const int i = threadIdx.x + c * blockDim.x;
-    const float d = i < H ? vals[c] - mean : 0.f;
-    ss = fmaf(d, d, ss);
+  for (int c = 0; c < G; ++c) {
+    const bool in = VEC * (threadIdx.x + c * blockDim.x) < H;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      const float d = in ? vals[c][e] - mean : 0.f;
+      ss = fmaf(d, d, ss);
+    }
   }
   ss = block_sum(ss, red);
   const float inv = 1.f / sqrtf(ss / (float)H + eps);
   float* xr = x + r * H;
 #pragma unroll
-  for (int c = 0; c < kNormAddPerThread; ++c) {
-    const int i = threadIdx.x + c * blockDim.x;
-    if (i < H) xr[i] += (vals[c] - mean) * inv * gain[gain_n == 1 ? 0 : i];
+  for (int c = 0; c < G; ++c) {
+    const int i = VEC * (threadIdx.x + c * blockDim.x);
+    if (i < H) {
+      float xv[VEC], gv[VEC];
+      na_load<VEC>(xr + i, xv);
+      if (gain_n == 1) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) gv[e] = gain[0];
+      } else {
+        na_load<VEC>(gain + i, gv);
+      }
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) xv[e] += (vals[c][e] - mean) * inv * gv[e];
+      if constexpr (VEC == 4) *(float4*)(xr + i) = make_float4(xv[0], xv[1], xv[2], xv[3]);
+      else xr[i] = xv[0];
+    }
   }
 }
 
@@ -200,11 +245,20 @@ extern "C" int ninfer_norm_add(float* x, const void* y, const float* gain, int g
   NINFER_REQUIRE(H <= 1024 * kNormAddPerThread, "norm_add: width %d exceeds %d", H,
                  1024 * kNormAddPerThread);
   NINFER_REQUIRE(!w || k > 0, "norm_add: a weighted sum of %d rows", k);
-  const int block = H >= 1024 ? 1024 : (H + 63) / 64 * 64;
-  if (dtype == kF32)
-    norm_add_kernel<float><<<T, block, 0, stream>>>(x, (const float*)y, w, k, gain, gain_n, H, eps, center);
-  else
-    norm_add_kernel<bf16><<<T, block, 0, stream>>>(x, (const bf16*)y, w, k, gain, gain_n, H, eps, center);
+  // groups of 4 consecutive numbers when every row stays 16-byte aligned
+  auto aligned = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+  const bool vec = H % 4 == 0 && aligned(x) && aligned(y) && (gain_n == 1 || aligned(gain));
+  const int per_thread = vec ? 4 : 1;
+  int block = ((H + per_thread - 1) / per_thread + 63) / 64 * 64;
+  if (block > 1024) block = 1024;
+  NINFER_REQUIRE((int64_t)block * kNormAddPerThread >= H, "norm_add: width %d exceeds the kernel's", H);
+  if (dtype == kF32) {
+    if (vec) norm_add_kernel<float, 4><<<T, block, 0, stream>>>(x, (const float*)y, w, k, gain, gain_n, H, eps, center);
+    else norm_add_kernel<float, 1><<<T, block, 0, stream>>>(x, (const float*)y, w, k, gain, gain_n, H, eps, center);
+  } else {
+    if (vec) norm_add_kernel<bf16, 4><<<T, block, 0, stream>>>(x, (const bf16*)y, w, k, gain, gain_n, H, eps, center);
+    else norm_add_kernel<bf16, 1><<<T, block, 0, stream>>>(x, (const bf16*)y, w, k, gain, gain_n, H, eps, center);
+  }
   NINFER_LAUNCH_CHECK();
   return 0;
 }

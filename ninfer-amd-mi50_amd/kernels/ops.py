@@ -95,7 +95,7 @@ class _QkvConvArgs(ctypes.Structure):
                 ("Hq", ctypes.c_int), ("Hkv", ctypes.c_int), ("dim", ctypes.c_int),
                 ("vdim", ctypes.c_int), ("taps", ctypes.c_int), ("rot_dim", ctypes.c_int),
                 ("interleaved", ctypes.c_int), ("page_size", ctypes.c_int),
-                ("dtype", ctypes.c_int), ("eps", ctypes.c_float)]
+                ("dtype", ctypes.c_int), ("eps", ctypes.c_float), ("all_single", ctypes.c_int)]
 
 
 class _QkvRopeArgs(ctypes.Structure):
@@ -924,7 +924,7 @@ class HipOps:
         if (ctx.max_qlen == 1 or single > 0) and qkv.dtype == torch.bfloat16 \
                 and not self.force_generic:
             ws_floats = int(self.lib.ninfer_attention_workspace_floats(
-                t if ctx.max_qlen == 1 else single, n_q, head_dim, ctx.max_kv_len))
+                t if ctx.max_qlen == 1 else single, n_q, max(head_dim, vdim), ctx.max_kv_len))
             if self._attn_ws is None or self._attn_ws.numel() < ws_floats:
                 # A captured graph may hold the address of the workspace it was recorded
                 # with: an outgrown one is kept, never given back (a replay would write
@@ -1009,6 +1009,7 @@ class HipOps:
         a.T, a.S, a.Hq, a.Hkv, a.dim, a.vdim, a.taps = t, ctx.S, heads, kv_heads, dim, vdim, taps
         a.rot_dim, a.interleaved, a.page_size = rot_dim, 1 if interleaved else 0, page_size
         a.dtype, a.eps = _DT[u.dtype], norm_eps
+        a.all_single = 1 if ctx.max_qlen == 1 else 0
         self._ok(self.lib.ninfer_qkv_conv(ctypes.byref(a), self._stream()))
 
     # ---- sublayers with the norm on their output -----------------------------------
