@@ -84,7 +84,8 @@ class _AttnArgs(ctypes.Structure):
 
 
 class _QkvConvArgs(ctypes.Structure):
-    _fields_ = [("u", ctypes.c_void_p), ("w", ctypes.c_void_p), ("state", ctypes.c_void_p),
+    _fields_ = [("u", ctypes.c_void_p), ("w", ctypes.c_void_p), ("wt", ctypes.c_void_p),
+                ("state", ctypes.c_void_p),
                 ("state_stride", ctypes.c_int64), ("q_out", ctypes.c_void_p),
                 ("kpool", ctypes.c_void_p), ("vpool", ctypes.c_void_p),
                 ("block_table", ctypes.c_void_p), ("positions", ctypes.c_void_p),
@@ -95,7 +96,8 @@ class _QkvConvArgs(ctypes.Structure):
                 ("Hq", ctypes.c_int), ("Hkv", ctypes.c_int), ("dim", ctypes.c_int),
                 ("vdim", ctypes.c_int), ("taps", ctypes.c_int), ("rot_dim", ctypes.c_int),
                 ("interleaved", ctypes.c_int), ("page_size", ctypes.c_int),
-                ("dtype", ctypes.c_int), ("eps", ctypes.c_float), ("all_single", ctypes.c_int)]
+                ("dtype", ctypes.c_int), ("eps", ctypes.c_float), ("all_single", ctypes.c_int),
+                ("force_plain", ctypes.c_int)]
 
 
 class _QkvRopeArgs(ctypes.Structure):
@@ -295,6 +297,7 @@ class HipOps:
         # (65: a decode step of up to 64 rows takes the same kernels run eagerly and captured)
         self.beside_heavy_min_rows = 65
         self.beside_heavy_bytes = 256 << 20
+        self.conv_pieces_always = False     # tests: qkv_conv's kernel of whole pieces at every row count
         self.gla_chunk_min_rows = 8         # the same for gated linear attention
         self.lightning_chunk_min_rows = 8   # a step's longest portion from which lightning attention runs in chunks
         self.library_min_rows = 32  # dense bf16 products with more rows go to the library
@@ -955,7 +958,7 @@ class HipOps:
 
     def qkv_conv(self, u, w_conv, state, ctx, q_out, heads, kv_heads, dim, vdim, k_pool, v_pool,
                  block_table, page_size, q_norm=None, k_norm=None, norm_eps=0.0, inv_freq=None,
-                 rot_dim=0, interleaved=False):
+                 rot_dim=0, interleaved=False, w_conv_t=None):
         """Projected rows u [T, heads * dim + kv_heads * (dim + vdim)] on their way to attention:
         a causal convolution over time per channel (`w_conv` [channels, taps], None: none; the
         taps - 1 projected rows before a step's first row come from `state` [slots, >= (taps - 1)
@@ -963,7 +966,9 @@ class HipOps:
         numbers (gains `q_norm`, `k_norm` [dim], None: no norm) and turned by their position
         (`inv_freq`, `rot_dim`, pairing as in `rope_kv_write`); queries to `q_out` [T, heads *
         dim], keys and values to the requests' pages of `k_pool` [pages, kv_heads, page_size,
-        dim] and `v_pool` [.., vdim]. kv_heads 0: the rows hold queries only."""
+        dim] and `v_pool` [.., vdim]. kv_heads 0: the rows hold queries only. `w_conv_t`: the
+        convolution's weights once more, transposed [taps, channels], for the kernel that moves
+        whole pieces of 8 channels (without it the kernel of a wave per head runs)."""
         _dev(u, "u", dims=2)
         _dev(q_out, "q_out", u.dtype, 2)
         t = ctx.T
@@ -978,6 +983,10 @@ class HipOps:
             taps = w_conv.shape[1]
             _need(w_conv.shape[0] == channels and taps >= 1, "qkv_conv: one row of taps per channel")
             a.w = w_conv.data_ptr()
+            if w_conv_t is not None:
+                _dev(w_conv_t, "w_conv_t", torch.float32, 2)
+                _need(w_conv_t.shape == (taps, channels), "qkv_conv: the transposed weights' shape")
+                a.wt = w_conv_t.data_ptr()
         if taps > 1:
             _need(state is not None and state.is_cuda and state.dtype == torch.float32
                   and state.dim() == 2 and state.stride(1) == 1
@@ -1010,6 +1019,7 @@ class HipOps:
         a.rot_dim, a.interleaved, a.page_size = rot_dim, 1 if interleaved else 0, page_size
         a.dtype, a.eps = _DT[u.dtype], norm_eps
         a.all_single = 1 if ctx.max_qlen == 1 else 0
+        a.force_plain = 1 if self.force_generic else 2 if self.conv_pieces_always else 0
         self._ok(self.lib.ninfer_qkv_conv(ctypes.byref(a), self._stream()))
 
     # ---- sublayers with the norm on their output -----------------------------------
@@ -1136,7 +1146,7 @@ class HipOps:
         a.positions, a.row_seq = ctx.positions.data_ptr(), ctx.row_seq.data_ptr()
         a.seq_row_start, a.seq_pos0 = ctx.seq_row_start.data_ptr(), ctx.seq_pos0.data_ptr()
         a.S, a.max_kv_len, a.max_qlen = ctx.S, ctx.max_kv_len, ctx.max_qlen
-        a.force_plain = 1 if self.force_generic else 0
+        a.force_plain = 1 if self.force_generic else 2 if self.conv_pieces_always else 0
         a.bt_stride, a.T, a.Hq, a.dim, a.R, a.rd, a.rot_n = \
             block_table.shape[1], ctx.T, heads, dim, rank, rot_dim, rot_n
         a.page_size, a.dtype = page_size, _DT[dtype]
@@ -1360,7 +1370,7 @@ class HipOps:
         a.q_stride, a.bt_stride, a.T, a.S = qkv.shape[1], block_table.shape[1], t, ctx.S
         a.Hq, a.Hkv, a.dim, a.vdim, a.page_size = heads, kv_heads, dim, vdim, page_size
         a.dtype, a.max_qlen, a.max_kv_len = _DT[qkv.dtype], ctx.max_qlen, ctx.max_kv_len
-        a.force_plain = 1 if self.force_generic else 0
+        a.force_plain = 1 if self.force_generic else 2 if self.conv_pieces_always else 0
         a.single_rows = int(getattr(ctx, "single_rows", 0))
         a.scale, a.cap, a.t_coef, a.t_every = scale, cap, temp_coef, int(temp_every)
         a.lam, a.eps, a.out_scale = lam, eps, out_scale
@@ -1517,7 +1527,7 @@ class HipOps:
         a.Hq, a.Hkv, a.dim, a.vdim, a.page_size = heads, kv_heads, dim, vdim, page_size
         a.dtype, a.max_qlen, a.max_kv_len = _DT[qkv.dtype], ctx.max_qlen, ctx.max_kv_len
         a.chunk, a.scale = int(chunk), float(scale)
-        a.force_plain = 1 if self.force_generic else 0
+        a.force_plain = 1 if self.force_generic else 2 if self.conv_pieces_always else 0
         a.single_rows = int(getattr(ctx, "single_rows", 0))
         if write_kv:
             self._ok(self.lib.ninfer_sigmoid_kv_write(ctypes.byref(a), self._stream()))

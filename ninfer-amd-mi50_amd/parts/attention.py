@@ -65,7 +65,8 @@ class Attention(Mixer):
         if self.general and qkv_bias:
             raise ValueError("q/k/v biases beside a convolution, values of their own size or "
                              "another layer's cache are not built")
-        self.w_conv: Optional[torch.Tensor] = None
+        self.w_conv: Optional[torch.Tensor] = None     # [channels, taps], as the checkpoint has it
+        self.w_conv_t: Optional[torch.Tensor] = None   # [taps, channels]: a tap's weights side by side
         if heads % kv_heads:
             raise ValueError(f"heads ({heads}) must be a multiple of kv_heads ({kv_heads})")
         if score_slopes is not None and len(score_slopes) != heads:
@@ -152,6 +153,7 @@ class Attention(Mixer):
             keys = ("q", "k", "v") if self.own_kv else ("q",)
             parts = [w.float32(p + n[key] + n["conv"]) for key in keys]
             self.w_conv = torch.cat(parts).contiguous()
+            self.w_conv_t = self.w_conv.t().contiguous()
             o = 0
             for key, part in zip(keys, parts):
                 w.hold(p + n[key] + n["conv"], self.w_conv[o:o + part.shape[0]])
@@ -179,7 +181,7 @@ class Attention(Mixer):
                      cache["v"], cache.block_table, cache.page_size, q_norm=self.q_norm,
                      k_norm=self.k_norm, norm_eps=self.qk_norm_eps or 0.0,
                      inv_freq=self.position.table(), rot_dim=self.position.rot_dim,
-                     interleaved=self.position.pairing == "interleaved")
+                     interleaved=self.position.pairing == "interleaved", w_conv_t=self.w_conv_t)
         attn = ctx.empty((ctx.T, self.heads * self.vdim))
         ops.paged_attention(q, cache["k"], cache["v"], cache.block_table, ctx, self.heads,
                             self.kv_heads, self.head_dim, cache.page_size, self.window, self.scale,

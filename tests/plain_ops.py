@@ -98,7 +98,7 @@ class PlainOps:
 
     def qkv_conv(self, u, w_conv, state, ctx, q_out, heads, kv_heads, dim, vdim, k_pool, v_pool,
                  block_table, page_size, q_norm=None, k_norm=None, norm_eps=0.0, inv_freq=None,
-                 rot_dim=0, interleaved=False):
+                 rot_dim=0, interleaved=False, w_conv_t=None):
         t, ch = u.shape
         y = _f(u).clone()
         if w_conv is not None:

@@ -110,15 +110,27 @@ def _gather(pool, table, n, page_size):
     return pool[pages, :, js % page_size, :]
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype,plain_kernel", [(torch.float32, False), (torch.bfloat16, False), (torch.bfloat16, True)])
 @pytest.mark.parametrize("heads,kv,dim,vdim,taps,rot,pairing", [
     (6, 3, 20, 12, 4, 10, "half"), (4, 2, 64, 32, 3, 64, "half"), (2, 1, 96, 80, 2, 48, "interleaved"),
-    (3, 0, 24, 8, 5, 24, "half"), (2, 2, 16, 16, 1, 0, "half"), (1, 1, 8, 40, 0, 8, "half")])
-def test_projected_rows_on_their_way_to_attention(ops, dtype, heads, kv, dim, vdim, taps, rot, pairing):
-    """Convolution, head norms, rotation and the cache write in one kernel: three requests in
-    slots 2, 0 and 3 of a wider state tensor, cut into portions down to two rows and single
-    rows (the taps - 1 rows before a portion come from the state), against the plain
-    convolution of the whole request followed by norm and rotation. kv 0: queries only."""
+    (3, 0, 24, 8, 5, 24, "half"), (2, 2, 16, 16, 1, 0, "half"), (1, 1, 8, 40, 0, 8, "half"),
+    (16, 4, 128, 128, 4, 64, "half")])
+def test_projected_rows_on_their_way_to_attention(ops, dtype, plain_kernel, heads, kv, dim, vdim, taps, rot, pairing):
+    """Convolution, head norms, rotation and the cache write in one kernel (a wave per head, or
+    for bfloat16 heads of whole pieces of 8 a thread per piece): three requests in slots 2, 0
+    and 3 of a wider state tensor, cut into portions down to two rows and single rows (the
+    taps - 1 rows before a portion come from the state), against the plain convolution of the
+    whole request followed by norm and rotation. kv 0: queries only."""
+    ops.force_generic = plain_kernel
+    ops.conv_pieces_always = not plain_kernel     # (the steps here have few rows)
+    try:
+        _projected_rows(ops, dtype, heads, kv, dim, vdim, taps, rot, pairing)
+    finally:
+        ops.force_generic = False
+        ops.conv_pieces_always = False
+
+
+def _projected_rows(ops, dtype, heads, kv, dim, vdim, taps, rot, pairing):
     g = torch.Generator().manual_seed(dim + taps)
     lens, ps, eps = [45, 7, 30], 8, 1e-5
     ch = heads * dim + kv * (dim + vdim)
@@ -147,7 +159,8 @@ def test_projected_rows_on_their_way_to_attention(ops, dtype, heads, kv, dim, vd
         q = torch.empty(ctx.T, heads * dim, dtype=dtype, device=DEV)
         ops.qkv_conv(u, w_conv.to(DEV) if taps else None, view, ctx, q, heads, kv, dim, vdim, k_pool, v_pool, bt,
                      ps, q_norm=qn.to(DEV), k_norm=kn.to(DEV) if kv else None, norm_eps=eps, inv_freq=freq,
-                     rot_dim=rot, interleaved=pairing == "interleaved")
+                     rot_dim=rot, interleaved=pairing == "interleaved",
+                     w_conv_t=w_conv.t().contiguous().to(DEV) if taps else None)
         o = 0
         for r, s, n in zip(who, starts, counts):
             got_q[r][s:s + n] = q[o:o + n].float().cpu()
@@ -563,6 +576,26 @@ def test_long_decoding(case, dtype):
     got = util.run_schedule(runner, util.schedule_tail("x", toks, n - 3))["x"]
     sub = {"name": case["name"], "ref": {dtype: {"x": ref}}, "noise": {dtype: {"x": noise_of(cfg, w, toks, ref)}}}
     check_logits(sub, dtype, {"x": got}, "long decoding")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_long_prompt(case, dtype):
+    """Hundreds of tokens in one step and in two portions (the kernels that many rows choose),
+    with keys far back for the layers that see them all."""
+    if case["name"] == "ones":
+        pytest.skip("covered by the other two")
+    from ninfer_amd import EngineOptions, load_model
+    n = 300
+    cfg, w = util.read_folder(case["dirs"][dtype])
+    toks = safe_prompt(w, cfg, n, 19)
+    ref = plain.forward(cfg, w, toks)[0]
+    sub = {"name": case["name"], "ref": {dtype: {"x": ref}}, "noise": {dtype: {"x": noise_of(cfg, w, toks, ref)}}}
+    runner = load_model(case["dirs"][dtype], EngineOptions(
+        dtype=dtype, max_context=320, prefill_chunk=320, num_sequences=2, page_size=16, num_pages=24,
+        check_pages=True, poison_freed_pages=True))
+    check_logits(sub, dtype, util.run_schedule(runner, util.schedule_whole("x", toks)), "whole")
+    steps = [([("x", toks[:257], list(range(257)))], []), ([("x", toks[257:], list(range(n - 257)))], ["x"])]
+    check_logits(sub, dtype, util.run_schedule(runner, steps), "two portions")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
