@@ -308,10 +308,16 @@ __global__ __launch_bounds__(128, 2) void attention_tiles_heads_kernel(AttnArgs 
   const int kt0 = first / 64 + ch * tiles_per_chunk;
   const int n_kt = min(pos / 64 + 1, kt0 + tiles_per_chunk);
   float* rec = n_chunks > 1 ? a.workspace + (((int64_t)t * a.Hq + h) * n_chunks + ch) * (2 + vdim) : nullptr;
-  if (kt0 >= n_kt) {   // nothing of this chunk is visible: records that count for nothing
-    if (q_valid && hi == 0 && kb == 0) {
-      rec[0] = -1e30f;
-      rec[1] = 0.f;
+  if (kt0 >= n_kt) {   // nothing of this chunk is visible: a record that counts for nothing
+    if (q_valid && kb == 0) {
+      if (hi == 0) {
+        rec[0] = -1e30f;
+        rec[1] = 0.f;
+      }
+      for (int col = 4 * hi; col < vdim; col += 8) {   // (a record starts at an even float: 8-byte stores)
+        *(float2*)(rec + 2 + col) = make_float2(0.f, 0.f);
+        *(float2*)(rec + 4 + col) = make_float2(0.f, 0.f);
+      }
     }
     return;
   }
@@ -415,25 +421,35 @@ __global__ __launch_bounds__(128, 2) void attention_tiles_heads_kernel(AttnArgs 
 }
 
 // The records of a row and head put together: out = sum_c o_c 2^(m_c - m) / sum_c l_c 2^(m_c - m).
+// Lane c weighs chunk c (64 chunks at a time); the outputs' loads do not wait for each other.
 __global__ __launch_bounds__(64) void attention_tiles_merge_kernel(AttnArgs a, int n_chunks) {
   const int th = blockIdx.x, lane = threadIdx.x;
-  const int vdim = a.Dv;
-  const float* rec = a.workspace + (int64_t)th * n_chunks * (2 + vdim);
+  const int vdim = a.Dv, stride = 2 + vdim;
+  const float* rec = a.workspace + (int64_t)th * n_chunks * stride;
   float mm = -1e30f;
-  for (int c = 0; c < n_chunks; ++c) mm = fmaxf(mm, rec[c * (2 + vdim)]);
+  for (int c = lane; c < n_chunks; c += 64) mm = fmaxf(mm, rec[c * stride]);
+  mm = wave_max(mm);
   float l = 0.f, acc[2] = {0.f, 0.f};
-  for (int c = 0; c < n_chunks; ++c) {
-    const float* r = rec + c * (2 + vdim);
-    if (r[1] == 0.f) continue;   // a chunk with no visible key holds no output
-    const float f = __builtin_amdgcn_exp2f(r[0] - mm);
-    l += r[1] * f;
+  for (int c0 = 0; c0 < n_chunks; c0 += 64) {
+    const int c = c0 + lane;
+    float f = 0.f;
+    if (c < n_chunks) {
+      f = __builtin_amdgcn_exp2f(rec[c * stride] - mm);
+      l += rec[c * stride + 1] * f;   // (a chunk with no visible key has l = 0 and o = 0)
+    }
+    const int cnt = min(64, n_chunks - c0);
+#pragma unroll 4
+    for (int j = 0; j < cnt; ++j) {
+      const float fj = __shfl(f, j, 64);
+      const float* r = rec + (c0 + j) * stride + 2;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int d = lane + 64 * i;
-      if (d < vdim) acc[i] += r[2 + d] * f;
+      for (int i = 0; i < 2; ++i) {
+        const int d = lane + 64 * i;
+        if (d < vdim) acc[i] = fmaf(r[d], fj, acc[i]);
+      }
     }
   }
-  const float inv = 1.f / l;
+  const float inv = 1.f / wave_sum(l);
   __bf16* orow = (__bf16*)a.out + (int64_t)th * vdim;
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
