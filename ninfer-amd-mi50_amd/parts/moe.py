@@ -212,6 +212,9 @@ class SparseMoE(FeedForward):
         self.identity = int(identity)
         if self.identity and shared_inner > 0:
             raise ValueError("identity experts beside a shared expert are not built")
+        if shared_inner > 0 and (router or {}).get("logit_bias_leaf"):
+            raise ValueError("a bias on the router's logits beside a shared expert is not built "
+                             "(the two share one product)")
         self.router = TopKRouter(prefix + n["router"], hidden, experts + self.identity, top_k,
                                  renorm, leaf=n["router_leaf"], weightless=self.identity,
                                  **(router or {}))
